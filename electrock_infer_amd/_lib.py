@@ -1,0 +1,106 @@
+"""ctypes binding of libelectrock_moe.so (the C ABI declared in include/electrock_moe.h).
+
+Nothing here computes: each wrapper turns torch tensors into raw device
+pointers plus the current HIP stream and raises RuntimeError on a non-zero
+status.  There is deliberately no CPU or eager-PyTorch fallback.
+"""
+import ctypes
+import os
+
+from ._build import LIB_PATH
+
+# element / index type codes of the C ABI
+DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
+ITYPE_I32, ITYPE_I64 = 0, 1
+
+FLAG_OUT_F32 = 1 << 0
+FLAG_SKIP_ROUTER = 1 << 8
+FLAG_SKIP_ALIGN = 1 << 9
+FLAG_SKIP_GEMM1 = 1 << 10
+FLAG_SKIP_GEMM2 = 1 << 11
+FLAG_SKIP_COMBINE = 1 << 12
+FLAG_FORCE_GENERIC = 1 << 16
+
+# every symbol include/electrock_moe.h declares
+EXPORTED_SYMBOLS = (
+    "em_version", "em_error_string", "em_topk_softmax", "em_moe_align_block_size",
+    "em_silu_and_mul", "em_moe_sum", "em_moe_workspace_bytes", "em_moe_workspace_layout",
+    "em_moe_forward",
+)
+
+
+class MoeLayout(ctypes.Structure):
+    """Mirror of struct em_moe_layout."""
+    _fields_ = [(n, ctypes.c_int64) for n in (
+        "block_size", "topk_weights_off", "topk_ids_off", "sorted_ids_off", "sorted_len",
+        "expert_ids_off", "expert_ids_len", "post_pad_off", "act_off", "y_off", "ksplit",
+        "total_bytes")]
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the built library; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m electrock_infer_amd._build` "
+            "(there is no fallback implementation)")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i32, i64, u32, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_uint, ctypes.c_size_t
+    lib.em_version.restype = i32
+    lib.em_version.argtypes = []
+    lib.em_error_string.restype = ctypes.c_char_p
+    lib.em_error_string.argtypes = [i32]
+    lib.em_topk_softmax.restype = i32
+    lib.em_topk_softmax.argtypes = [vp, i32, i64, i32, i32, i32, vp, vp, vp]
+    lib.em_moe_align_block_size.restype = i32
+    lib.em_moe_align_block_size.argtypes = [vp, i32, i64, i32, i32, vp, i64, vp, i64, vp, vp]
+    lib.em_silu_and_mul.restype = i32
+    lib.em_silu_and_mul.argtypes = [vp, vp, i64, i64, i32, vp]
+    lib.em_moe_sum.restype = i32
+    lib.em_moe_sum.argtypes = [vp, vp, i64, i32, i64, i32, vp]
+    lib.em_moe_workspace_bytes.restype = sz
+    lib.em_moe_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
+    lib.em_moe_workspace_layout.restype = i32
+    lib.em_moe_workspace_layout.argtypes = [i64, i32, i32, i32, i32, ctypes.POINTER(MoeLayout)]
+    lib.em_moe_forward.restype = i32
+    lib.em_moe_forward.argtypes = [vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().em_error_string(code).decode()
+        raise RuntimeError(f"{what} failed: {msg} (status {code})")
+
+
+def dtype_code(dtype) -> int:
+    import torch
+    try:
+        return {torch.float32: DTYPE_F32, torch.bfloat16: DTYPE_BF16, torch.float16: DTYPE_F16}[dtype]
+    except KeyError:
+        raise RuntimeError(f"unsupported element type {dtype}") from None
+
+
+def current_stream(device) -> int:
+    import torch
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_device(*tensors) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("tensor must be on a GPU device (no CPU path exists)")
+        if not t.is_contiguous():
+            raise RuntimeError("tensor must be contiguous")
+
+
+def workspace_layout(T: int, H: int, I: int, E: int, top_k: int) -> MoeLayout:
+    L = MoeLayout()
+    check(load().em_moe_workspace_layout(T, H, I, E, top_k, ctypes.byref(L)), "em_moe_workspace_layout")
+    return L

@@ -1,0 +1,124 @@
+// Expert sort (moe_align_block_size): stable counting sort of the flat slot
+// indices by expert, every expert segment padded to a multiple of block_size.
+//
+// One workgroup of 16 wavefronts.  Wave w owns the contiguous chunk
+// [w*chunk, (w+1)*chunk) of topk_ids:
+//   pass 1  per-wave histogram with ballots           -> LDS hist[wave][expert]
+//   scan    exclusive prefix over waves per expert, padded exclusive prefix
+//           over experts                               -> LDS base[wave][expert]
+//   pass 2  each wave re-walks its chunk; lane e keeps the running write
+//           position of expert e, a slot's position is that value (read with a
+//           lane shuffle) plus its rank among equal experts in the 64-wide step.
+// Chunks are contiguous and walked in ascending order, so the sort is stable,
+// as the reference's per-thread chunks are (src/moe_align_block_size.hip:78-135).
+// Output conventions follow the reference wrapper
+// (layers/moe/moe_align_block_size.py:32-48): pads and tail of sorted ids are -1,
+// unused tail of expert_ids is 0.
+#include "common.h"
+
+namespace em {
+namespace {
+
+constexpr int kAlignThreads = 1024;
+constexpr int kAlignWaves = kAlignThreads / kWave;
+
+template <typename IdT>
+__global__ __launch_bounds__(kAlignThreads) void align_kernel(
+    const IdT* __restrict__ ids, int64_t numel, int E, int block,
+    int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
+    int64_t eid_len, int32_t* __restrict__ post_pad) {
+    __shared__ int32_t hist[kAlignWaves][kMaxExperts];  // pass 1 counts, then write bases
+    __shared__ int32_t seg_begin[kMaxExperts + 1];      // padded exclusive prefix
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
+
+    const int64_t chunk = round_up(ceil_div(numel, kAlignWaves), kWave);
+    const int64_t begin = wave * chunk;
+    const int64_t end = (begin + chunk < numel) ? begin + chunk : numel;
+
+    // every output element is defined by this kernel: start from the pad values
+    for (int64_t i = tid; i < sorted_len; i += kAlignThreads) sorted[i] = -1;
+    for (int64_t i = tid; i < eid_len; i += kAlignThreads) expert_ids[i] = 0;
+
+    // ---- pass 1: per-wave histogram (lane e accumulates expert e) ----
+    int32_t cnt = 0;
+    for (int64_t i0 = begin; i0 < end; i0 += kWave) {
+        const int64_t i = i0 + lane;
+        const int e = (i < end) ? static_cast<int>(ids[i]) : -1;
+        for (int j = 0; j < E; ++j) {
+            const uint64_t m = __ballot(e == j);
+            if (lane == j) cnt += __popcll(m);
+        }
+    }
+    if (lane < kMaxExperts) hist[wave][lane] = (lane < E) ? cnt : 0;
+    __syncthreads();
+
+    // ---- scan: thread e turns counts into per-wave write bases ----
+    int32_t total = 0;
+    if (tid < E) {
+        for (int w = 0; w < kAlignWaves; ++w) {
+            const int32_t c = hist[w][tid];
+            hist[w][tid] = total;  // exclusive prefix over waves
+            total += c;
+        }
+        seg_begin[tid + 1] = static_cast<int32_t>(round_up(total, block));
+    }
+    if (tid == 0) seg_begin[0] = 0;
+    __syncthreads();
+    if (tid == 0) {
+        int32_t run = 0;
+        for (int e = 0; e < E; ++e) {
+            const int32_t padded = seg_begin[e + 1];
+            seg_begin[e] = run;
+            run += padded;
+        }
+        seg_begin[E] = run;
+        post_pad[0] = run;
+    }
+    __syncthreads();  // also orders the -1 / 0 fill before the scatter below
+
+    // block -> expert table
+    if (tid < E) {
+        for (int32_t p = seg_begin[tid]; p < seg_begin[tid + 1]; p += block)
+            if (p / block < eid_len) expert_ids[p / block] = tid;
+    }
+
+    // ---- pass 2: stable scatter ----
+    int32_t pos = (lane < E) ? seg_begin[lane] + hist[wave][lane] : 0;
+    for (int64_t i0 = begin; i0 < end; i0 += kWave) {
+        const int64_t i = i0 + lane;
+        const int e = (i < end) ? static_cast<int>(ids[i]) : -1;
+        const bool valid = (e >= 0 && e < E);
+        const int32_t base = __shfl(pos, valid ? e : 0);
+        int32_t rank = 0;
+        for (int j = 0; j < E; ++j) {
+            const uint64_t m = __ballot(e == j);
+            if (e == j) rank = __popcll(m & lt_mask);
+            if (lane == j) pos += __popcll(m);
+        }
+        if (valid && base + rank < sorted_len) sorted[base + rank] = static_cast<int32_t>(i);
+    }
+}
+
+}  // namespace
+
+int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
+                 int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
+                 int32_t* post_pad, hipStream_t s) {
+    const dim3 grid(1), blk(kAlignThreads);
+    if (itype == EM_ITYPE_I32) {
+        hipLaunchKernelGGL(align_kernel<int32_t>, grid, blk, 0, s, static_cast<const int32_t*>(ids),
+                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad);
+    } else if (itype == EM_ITYPE_I64) {
+        hipLaunchKernelGGL(align_kernel<int64_t>, grid, blk, 0, s, static_cast<const int64_t*>(ids),
+                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad);
+    } else {
+        return EM_ERR_BAD_DTYPE;
+    }
+    return launch_status();
+}
+
+}  // namespace em

@@ -1,0 +1,187 @@
+// extern "C" surface of libelectrock_moe.so: argument checks, workspace layout
+// and stage sequencing.  No kernel code lives here.
+#include "common.h"
+
+using namespace em;
+
+namespace {
+
+constexpr int kVersion = 100;
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+inline bool dtype_ok(int d) { return d == EM_DTYPE_F32 || d == EM_DTYPE_BF16 || d == EM_DTYPE_F16; }
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Counterpart of _get_moe_config (fused_moe.py:327-339): rows per sorted block.
+// An expert receives at most T rows, so up to 16 tokens one 16-row MFMA
+// fragment per expert always suffices; above that one 64-row block per expert
+// keeps each weight tile read by a single workgroup for decode batches.
+inline int choose_block(int64_t T) { return T <= 16 ? 16 : 64; }
+// Split of the w2 reduction (K = I) across workgroups for small batches, where
+// (row blocks) x (H / 128 column tiles) alone would leave most CUs idle.
+inline int choose_ksplit(int64_t T) { return T <= 64 ? 8 : (T <= 512 ? 4 : 1); }
+
+bool shapes_ok(int64_t T, int H, int I, int E, int top_k) {
+    return T >= 0 && H > 0 && I > 0 && E >= 1 && E <= kMaxExperts && top_k >= 1 && top_k <= kMaxTopK &&
+           top_k <= E && H % 8 == 0 && I % 8 == 0 && T * top_k < (int64_t(1) << 30);
+}
+
+}  // namespace
+
+extern "C" {
+
+int em_version(void) { return kVersion; }
+
+const char* em_error_string(int code) {
+    switch (code) {
+        case 0: return "success";
+        case EM_ERR_NULL_POINTER: return "null pointer argument";
+        case EM_ERR_BAD_SHAPE: return "invalid shape argument";
+        case EM_ERR_BAD_DTYPE: return "unsupported element type";
+        case EM_ERR_UNSUPPORTED: return "configuration not supported by this build";
+        case EM_ERR_WORKSPACE: return "workspace too small";
+        case EM_ERR_BUFFER_SIZE: return "output buffer too small";
+        case EM_ERR_ALIGNMENT: return "pointer not sufficiently aligned";
+        default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
+    }
+}
+
+int em_topk_softmax(const void* logits, int logits_dtype, int64_t T, int E, int k, int renormalize,
+                    float* topk_weights, int32_t* topk_ids, void* stream) {
+    if (T < 0 || E < 1 || E > kMaxExperts || k < 1 || k > E) return EM_ERR_BAD_SHAPE;
+    if (!dtype_ok(logits_dtype)) return EM_ERR_BAD_DTYPE;
+    if (T == 0) return 0;
+    if (!logits || !topk_weights || !topk_ids) return EM_ERR_NULL_POINTER;
+    return launch_router(logits, logits_dtype, T, E, k, renormalize, topk_weights, topk_ids, as_stream(stream));
+}
+
+int em_moe_align_block_size(const void* topk_ids, int ids_itype, int64_t numel, int num_experts,
+                            int block_size, int32_t* sorted_token_ids, int64_t sorted_len,
+                            int32_t* expert_ids, int64_t expert_ids_len, int32_t* num_tokens_post_pad,
+                            void* stream) {
+    if (numel < 0 || num_experts < 1 || num_experts > kMaxExperts || block_size < 1 ||
+        numel >= (int64_t(1) << 30))
+        return EM_ERR_BAD_SHAPE;
+    if (ids_itype != EM_ITYPE_I32 && ids_itype != EM_ITYPE_I64) return EM_ERR_BAD_DTYPE;
+    if (!sorted_token_ids || !expert_ids || !num_tokens_post_pad || (numel > 0 && !topk_ids))
+        return EM_ERR_NULL_POINTER;
+    if (sorted_len < 0 || expert_ids_len < 0) return EM_ERR_BUFFER_SIZE;
+    return launch_align(topk_ids, ids_itype, numel, num_experts, block_size, sorted_token_ids, sorted_len,
+                        expert_ids, expert_ids_len, num_tokens_post_pad, as_stream(stream));
+}
+
+int em_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, void* stream) {
+    if (rows < 0 || d < 0 || rows >= (int64_t(1) << 31)) return EM_ERR_BAD_SHAPE;
+    if (!dtype_ok(dtype)) return EM_ERR_BAD_DTYPE;
+    if (rows == 0 || d == 0) return 0;
+    if (!out || !in) return EM_ERR_NULL_POINTER;
+    return launch_silu_and_mul(out, in, rows, d, dtype, as_stream(stream));
+}
+
+int em_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype, void* stream) {
+    if (T < 0 || H < 0 || topk < 1 || T >= (int64_t(1) << 31)) return EM_ERR_BAD_SHAPE;
+    if (!dtype_ok(dtype)) return EM_ERR_BAD_DTYPE;
+    if (T == 0 || H == 0) return 0;
+    if (!out || !in) return EM_ERR_NULL_POINTER;
+    return launch_moe_sum(in, out, T, topk, H, dtype, as_stream(stream));
+}
+
+int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_layout* L) {
+    if (!L) return EM_ERR_NULL_POINTER;
+    if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
+    const int64_t block = choose_block(T);
+    const int64_t slots = T * top_k;
+    const int64_t sorted_len = round_up(slots + static_cast<int64_t>(E) * (block - 1), block);
+    int64_t off = 0;
+    auto take = [&off](int64_t bytes) {
+        const int64_t at = off;
+        off += round_up(bytes > 0 ? bytes : 1, 256);
+        return at;
+    };
+    L->block_size = block;
+    L->topk_weights_off = take(slots * 4);
+    L->topk_ids_off = take(slots * 4);
+    L->sorted_ids_off = take(sorted_len * 4);
+    L->sorted_len = sorted_len;
+    L->expert_ids_len = sorted_len / block;
+    L->expert_ids_off = take(L->expert_ids_len * 4);
+    L->post_pad_off = take(4);
+    L->act_off = take(sorted_len * static_cast<int64_t>(I) * 2);
+    L->ksplit = choose_ksplit(T);
+    L->y_off = take(L->ksplit * slots * static_cast<int64_t>(H) * 4);
+    L->total_bytes = off;
+    return 0;
+}
+
+size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k) {
+    em_moe_layout L;
+    if (em_moe_workspace_layout(T, H, I, E, top_k, &L) != 0) return 0;
+    return static_cast<size_t>(L.total_bytes);
+}
+
+int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, const void* w13,
+                   const void* w2, void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
+                   void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
+    if (!dtype_ok(logits_dtype)) return EM_ERR_BAD_DTYPE;
+    if (T == 0) return 0;
+    if (!x || !router_logits || !w13 || !w2 || !out || !workspace) return EM_ERR_NULL_POINTER;
+    if (!aligned(x, 16) || !aligned(w13, 16) || !aligned(w2, 16) || !aligned(out, 16) ||
+        !aligned(workspace, 256))
+        return EM_ERR_ALIGNMENT;
+    em_moe_layout L;
+    int rc = em_moe_workspace_layout(T, H, I, E, top_k, &L);
+    if (rc != 0) return rc;
+    if (workspace_bytes < static_cast<size_t>(L.total_bytes)) return EM_ERR_WORKSPACE;
+
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    hipStream_t s = as_stream(stream);
+    MoeProblem p;
+    p.x = static_cast<const uint16_t*>(x);
+    p.w13 = static_cast<const uint16_t*>(w13);
+    p.w2 = static_cast<const uint16_t*>(w2);
+    p.act = reinterpret_cast<uint16_t*>(ws + L.act_off);
+    p.y = reinterpret_cast<float*>(ws + L.y_off);
+    int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
+    int32_t* eids = reinterpret_cast<int32_t*>(ws + L.expert_ids_off);
+    int32_t* post_pad = reinterpret_cast<int32_t*>(ws + L.post_pad_off);
+    float* topk_w = reinterpret_cast<float*>(ws + L.topk_weights_off);
+    int32_t* topk_ids = reinterpret_cast<int32_t*>(ws + L.topk_ids_off);
+    p.sorted_ids = sorted;
+    p.expert_ids = eids;
+    p.post_pad = post_pad;
+    p.topk_w = topk_w;
+    p.T = T;
+    p.H = H;
+    p.I = I;
+    p.E = E;
+    p.top_k = top_k;
+    p.block = static_cast<int>(L.block_size);
+    p.sorted_len = L.sorted_len;
+    p.ksplit = static_cast<int>(L.ksplit);
+
+    if (!(flags & EM_FLAG_SKIP_ROUTER)) {
+        rc = launch_router(router_logits, logits_dtype, T, E, top_k, renormalize, topk_w, topk_ids, s);
+        if (rc != 0) return rc;
+    }
+    if (!(flags & EM_FLAG_SKIP_ALIGN)) {
+        rc = launch_align(topk_ids, EM_ITYPE_I32, T * top_k, E, p.block, sorted, L.sorted_len, eids,
+                          L.expert_ids_len, post_pad, s);
+        if (rc != 0) return rc;
+    }
+    if (!(flags & EM_FLAG_SKIP_GEMM1)) {
+        rc = launch_gemm_generic(p, 1, s);
+        if (rc != 0) return rc;
+    }
+    if (!(flags & EM_FLAG_SKIP_GEMM2)) {
+        rc = launch_gemm_generic(p, 2, s);
+        if (rc != 0) return rc;
+    }
+    if (!(flags & EM_FLAG_SKIP_COMBINE)) {
+        rc = launch_combine(p, out, (flags & EM_FLAG_OUT_F32) ? 1 : 0, s);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+// Shared device/host helpers for the gfx950 MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/electrock_moe.h"
+
+namespace em {
+
+constexpr int kWave = 64;          // CDNA wavefront width
+constexpr int kMaxExperts = 64;    // one lane per expert in the router / sort
+constexpr int kMaxTopK = 8;
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__host__ __device__ constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__host__ __device__ constexpr int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+
+// ---- bf16 / f16 <-> f32 on raw bits (round to nearest even) -----------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+    return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);  // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return static_cast<float>(v);
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    _Float16 v = static_cast<_Float16>(f);
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+// two packed bf16 in one dword
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return static_cast<uint32_t>(f32_to_bf16_bits(lo)) | (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
+}
+
+// Element traits for the three storage types the ops accept.
+struct F32Elem {
+    typedef float storage;
+    static __device__ __forceinline__ float load(const storage& v) { return v; }
+    static __device__ __forceinline__ storage store(float f) { return f; }
+};
+struct BF16Elem {
+    typedef uint16_t storage;
+    static __device__ __forceinline__ float load(const storage& v) { return bf16_bits_to_f32(v); }
+    static __device__ __forceinline__ storage store(float f) { return f32_to_bf16_bits(f); }
+};
+struct F16Elem {
+    typedef uint16_t storage;
+    static __device__ __forceinline__ float load(const storage& v) { return f16_bits_to_f32(v); }
+    static __device__ __forceinline__ storage store(float f) { return f32_to_f16_bits(f); }
+};
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+inline int launch_status() { return static_cast<int>(hipGetLastError()); }
+
+// ---- stage launchers (defined in the .hip files, called from capi.hip) ------
+int launch_router(const void* logits, int logits_dtype, int64_t T, int E, int k, int renorm,
+                  float* w, int32_t* ids, hipStream_t s);
+int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
+                 int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
+                 int32_t* post_pad, hipStream_t s);
+int launch_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, hipStream_t s);
+int launch_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype, hipStream_t s);
+
+// Problem description shared by the expert GEMM stages.
+struct MoeProblem {
+    const uint16_t* x;        // [T, H] bf16
+    const uint16_t* w13;      // [E, 2I, H] bf16
+    const uint16_t* w2;       // [E, H, I] bf16
+    uint16_t* act;            // [sorted_len, I] bf16, rows in sorted (padded) order
+    float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
+    const int32_t* sorted_ids;
+    const int32_t* expert_ids;
+    const int32_t* post_pad;
+    const float* topk_w;      // [T*top_k]
+    int64_t T;
+    int H, I, E, top_k;
+    int block;                // rows per sorted block
+    int64_t sorted_len;       // worst-case padded length
+    int ksplit;
+};
+int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s);  // mode 1: w13+SiLU*mul, 2: w2
+int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s);
+
+}  // namespace em

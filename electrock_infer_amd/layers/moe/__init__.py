@@ -1,0 +1,3 @@
+from .fused_moe import fused_experts, fused_topk  # noqa: F401
+from .mixtral_moe import FusedMoE  # noqa: F401
+from .moe_align_block_size import moe_align_block_size  # noqa: F401

@@ -1,0 +1,140 @@
+"""Host side of the MoE hot path, mirroring
+electrock_infer/layers/moe/fused_moe.py of the reference.
+
+``fused_topk`` and ``fused_experts`` keep the reference's names, argument
+meaning and return values; behind them sits one call into the C ABI
+(``em_topk_softmax`` / ``em_moe_forward``) instead of torch ops + Triton.
+"""
+import ctypes
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from ... import _lib
+
+
+def _get_moe_config(num_tokens: int, num_experts: int, intermediate_size: int, topk: int) -> dict:
+    """Row-block size of the expert sort as the reference picks it
+    (fused_moe.py:327-339).  Kept for callers that run the ops one by one; the
+    fused entry point chooses its own tiling (see ``workspace_layout``)."""
+    if num_tokens <= num_experts:
+        return {"BLOCK_SIZE_M": 16, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
+    return {"BLOCK_SIZE_M": 64, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
+
+
+def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int,
+               renormalize: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Softmax + top-k (+ renormalise) of the router logits
+    (fused_moe.py:130-164).  Returns float32 weights and int32 expert ids;
+    ties go to the lowest expert index."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    _lib.require_device(gating_output)
+    M, E = gating_output.shape
+    topk_weights = torch.empty(M, topk, dtype=torch.float32, device=gating_output.device)
+    topk_ids = torch.empty(M, topk, dtype=torch.int32, device=gating_output.device)
+    code = _lib.load().em_topk_softmax(gating_output.data_ptr(), _lib.dtype_code(gating_output.dtype), M, E,
+                                       topk, 1 if renormalize else 0, topk_weights.data_ptr(),
+                                       topk_ids.data_ptr(), _lib.current_stream(gating_output.device))
+    _lib.check(code, "fused_topk")
+    return topk_weights, topk_ids
+
+
+class MoeWorkspace:
+    """Device scratch for ``em_moe_forward``, cached per (device, shape).
+
+    The reference allocates its three intermediate caches and the sort buffers
+    on every call (fused_moe.py:223-239, moe_align_block_size.py:32-48); here one
+    256-byte aligned buffer is kept and reused, and views of the routing results
+    the kernels leave in it can be read back for inspection.
+    """
+
+    def __init__(self, device, T: int, H: int, I: int, E: int, top_k: int):
+        self.shape = (T, H, I, E, top_k)
+        self.layout = _lib.workspace_layout(T, H, I, E, top_k)
+        self.buffer = torch.empty(self.layout.total_bytes, dtype=torch.uint8, device=device)
+        assert self.buffer.data_ptr() % 256 == 0
+
+    def _view(self, off: int, count: int, dtype: torch.dtype) -> torch.Tensor:
+        nbytes = count * torch.empty((), dtype=dtype).element_size()
+        return self.buffer[off:off + nbytes].view(dtype)
+
+    @property
+    def block_size(self) -> int:
+        return self.layout.block_size
+
+    def topk_weights(self) -> torch.Tensor:
+        T, _, _, _, k = self.shape
+        return self._view(self.layout.topk_weights_off, T * k, torch.float32).view(T, k)
+
+    def topk_ids(self) -> torch.Tensor:
+        T, _, _, _, k = self.shape
+        return self._view(self.layout.topk_ids_off, T * k, torch.int32).view(T, k)
+
+    def sorted_token_ids(self) -> torch.Tensor:
+        return self._view(self.layout.sorted_ids_off, self.layout.sorted_len, torch.int32)
+
+    def expert_ids(self) -> torch.Tensor:
+        return self._view(self.layout.expert_ids_off, self.layout.expert_ids_len, torch.int32)
+
+    def num_tokens_post_pad(self) -> torch.Tensor:
+        return self._view(self.layout.post_pad_off, 1, torch.int32)
+
+
+_workspaces: Dict[tuple, MoeWorkspace] = {}
+
+
+def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int) -> MoeWorkspace:
+    key = (torch.device(device).index, T, H, I, E, top_k)
+    ws = _workspaces.get(key)
+    if ws is None:
+        # keep one workspace per device: drop those of other batch sizes
+        for k in [k for k in _workspaces if k[0] == key[0]]:
+            del _workspaces[k]
+        ws = _workspaces[key] = MoeWorkspace(device, T, H, I, E, top_k)
+    return ws
+
+
+def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                  gating_output: torch.Tensor, topk: int, renormalize: bool = True,
+                  inplace: bool = False, activation: str = "silu",
+                  out_dtype: Optional[torch.dtype] = None, flags: int = 0,
+                  workspace: Optional[MoeWorkspace] = None) -> torch.Tensor:
+    """The MoE layer body (fused_moe.py:170-293): route, sort, w13 GEMM with
+    SiLU*mul, w2 GEMM, weighted top-k combine.
+
+    hidden_states [T, H] bf16; w1 [E, 2I, H] (gate rows then up rows); w2 [E, H, I];
+    gating_output [T, E].  With ``inplace`` the result overwrites
+    ``hidden_states`` and that tensor is returned, as in the reference.
+    ``out_dtype=torch.float32`` returns the un-rounded fp32 result instead
+    (not available together with ``inplace``).
+    """
+    if activation != "silu":
+        raise NotImplementedError(f"Activation {activation} not supported.")
+    _lib.require_device(hidden_states, w1, w2, gating_output)
+    T, H = hidden_states.shape
+    E, two_i, Hw = w1.shape
+    I = two_i // 2
+    if Hw != H or tuple(w2.shape) != (E, H, I) or two_i != 2 * I:
+        raise RuntimeError("weight shapes do not match hidden_states")
+    if gating_output.shape[0] != T or gating_output.shape[1] != E:
+        raise RuntimeError("gating_output must be [num_tokens, num_experts]")
+    if not (hidden_states.dtype == w1.dtype == w2.dtype == torch.bfloat16):
+        raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, w1 and w2 must be bfloat16")
+    want_f32 = out_dtype == torch.float32
+    if want_f32 and inplace:
+        raise RuntimeError("a float32 result cannot be written in place over bfloat16 hidden_states")
+    if want_f32:
+        output = torch.empty((T, H), dtype=torch.float32, device=hidden_states.device)
+        flags |= _lib.FLAG_OUT_F32
+    else:
+        output = hidden_states if inplace else torch.empty_like(hidden_states)
+    if T == 0:
+        return output
+    ws = workspace or get_workspace(hidden_states.device, T, H, I, E, topk)
+    code = _lib.load().em_moe_forward(
+        hidden_states.data_ptr(), gating_output.data_ptr(), _lib.dtype_code(gating_output.dtype),
+        w1.data_ptr(), w2.data_ptr(), output.data_ptr(), T, H, I, E, topk, 1 if renormalize else 0,
+        ws.buffer.data_ptr(), ctypes.c_size_t(ws.buffer.numel()), flags,
+        _lib.current_stream(hidden_states.device))
+    _lib.check(code, "fused_experts")
+    return output

@@ -1,0 +1,174 @@
+/*
+ * electrock_moe.h — C ABI of libelectrock_moe.so (MI355X / gfx950).
+ *
+ * Drop-in boundary for the Mixtral MoE layer of RouteTrace/electrock-infer.
+ * Every entry point takes raw DEVICE pointers, plain sizes and a HIP stream
+ * (passed as void* so that this header needs no HIP include), launches
+ * asynchronously on that stream, never allocates, frees or retains memory and
+ * keeps no mutable global state.  The caller guarantees that the device owning
+ * the pointers is current.
+ *
+ * Return value of every function returning int:
+ *     0   success (work is queued on `stream`)
+ *   < 0   argument error, nothing was launched (EM_ERR_*)
+ *   > 0   a hipError_t reported by the runtime after the launch
+ *
+ * Citations are relative to the reference tree (RouteTrace/electrock-infer).
+ */
+#ifndef ELECTROCK_MOE_H
+#define ELECTROCK_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type codes */
+#define EM_DTYPE_F32  0
+#define EM_DTYPE_BF16 1
+#define EM_DTYPE_F16  2
+/* index type codes (topk_ids) */
+#define EM_ITYPE_I32  0
+#define EM_ITYPE_I64  1
+
+/* argument errors */
+#define EM_ERR_NULL_POINTER   (-1)
+#define EM_ERR_BAD_SHAPE      (-2)
+#define EM_ERR_BAD_DTYPE      (-3)
+#define EM_ERR_UNSUPPORTED    (-4)
+#define EM_ERR_WORKSPACE      (-5)
+#define EM_ERR_BUFFER_SIZE    (-6)
+#define EM_ERR_ALIGNMENT      (-7)
+
+/* em_moe_forward flags */
+#define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16      */
+#define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
+#define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
+#define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
+#define EM_FLAG_SKIP_GEMM2     (1u << 11)
+#define EM_FLAG_SKIP_COMBINE   (1u << 12)
+#define EM_FLAG_FORCE_GENERIC  (1u << 16) /* use the shape-generic GEMM kernels           */
+
+/* Library version, e.g. 100 = 0.1.0. */
+int em_version(void);
+
+/* Human-readable text for a return code of this library (static storage). */
+const char* em_error_string(int code);
+
+/*
+ * Router: row-wise softmax + top-k (+ optional renormalisation).
+ * Replaces  _C.topk_softmax(topk_weights, topk_indices, gating_output)
+ *   (pytorch_bind.cpp:24-29, src/topk_softmax_kernels.hip:11-114) and, with
+ *   renormalize=1, fused_topk (electrock_infer/layers/moe/fused_moe.py:130-164).
+ * Selection compares raw logits; ties go to the LOWEST expert index
+ * (strict '>' scan, topk_softmax_kernels.hip:42-55).  topk_ids[:,0] is the arg-max.
+ *   logits        [T, E]  logits_dtype in {F32, BF16, F16}, row-major
+ *   topk_weights  [T, k]  float32   softmax probability (divided by the sum of
+ *                                   the k selected ones when renormalize != 0)
+ *   topk_ids      [T, k]  int32
+ * Limits: 1 <= k <= E <= 64.
+ */
+int em_topk_softmax(const void* logits, int logits_dtype, int64_t T, int E, int k,
+                    int renormalize, float* topk_weights, int32_t* topk_ids,
+                    void* stream);
+
+/*
+ * Expert sort with padding to the GEMM block size.
+ * Replaces  _C.moe_align_block_size(topk_ids, num_experts, block_size,
+ *                                   sorted_token_ids, expert_ids, num_tokens_post_pad)
+ *   (pytorch_bind.cpp:43-51, src/moe_align_block_size.hip:61-233) together with
+ *   the buffer conventions of its wrapper
+ *   (electrock_infer/layers/moe/moe_align_block_size.py:32-60):
+ *   sorted_token_ids  [sorted_len]  int32, flat slot indices i = t*k + j grouped by
+ *                     expert, ascending inside an expert, every expert segment padded
+ *                     to a multiple of block_size with -1; everything after
+ *                     num_tokens_post_pad is -1 too
+ *   expert_ids        [expert_ids_len] int32, expert of each block; unused tail = 0
+ *   num_tokens_post_pad [1] int32, sum over experts of ceil(cnt/block)*block
+ * The kernel writes EVERY element of the three outputs, so it needs no
+ * pre-filled buffers and yields identical bytes on pre-filled ones.
+ * sorted_len >= numel + E*(block_size-1) and expert_ids_len >= ceil(that / block_size)
+ * always suffice (the wrapper's sizes); shorter buffers are legal when the caller
+ * knows the padded total (the reference's own test sizes them exactly,
+ * test/example/test_align_block.py:142-147): writes never go past the given lengths.
+ * Entries of topk_ids outside [0, E) are ignored.   Limits: 1 <= E <= 64.
+ */
+int em_moe_align_block_size(const void* topk_ids, int ids_itype, int64_t numel,
+                            int num_experts, int block_size,
+                            int32_t* sorted_token_ids, int64_t sorted_len,
+                            int32_t* expert_ids, int64_t expert_ids_len,
+                            int32_t* num_tokens_post_pad, void* stream);
+
+/*
+ * out[r, j] = T( T(silu_f32(in[r, j])) * in[r, d + j] ),  r < rows, j < d.
+ * Replaces  _C.silu_and_mul(out, input)
+ *   (pytorch_bind.cpp:18-22, src/activation_kernels.hip:23-47,99-152).
+ *   in [rows, 2d], out [rows, d], same dtype in {F32, BF16, F16}.
+ */
+int em_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype,
+                    void* stream);
+
+/*
+ * out[t, j] = sum over kk < topk of in[t, kk, j], accumulated in the element
+ * type in ascending kk.
+ * Replaces  _C.moe_sum(input, output)
+ *   (pytorch_bind.cpp:31-35, src/moe_sum.hip:30-77).
+ *   in [T, topk, H], out [T, H], same dtype in {F32, BF16, F16}.
+ */
+int em_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype,
+               void* stream);
+
+/*
+ * Bytes of device workspace em_moe_forward needs for these shapes
+ * (0 for invalid shapes).  The workspace must be 256-byte aligned.
+ */
+size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
+
+/*
+ * The whole layer:  out[t] = sum_j w[t,j] * W2[e_tj] ( silu(W1[e_tj] x_t) * (W3[e_tj] x_t) ).
+ * Replaces  fused_experts(hidden_states, w1, w2, gating_output, topk, renormalize,
+ *                         inplace, "silu")
+ *   (electrock_infer/layers/moe/fused_moe.py:170-293) as called by FusedMoE.forward
+ *   (electrock_infer/layers/moe/mixtral_moe.py:100-109).
+ *   x             [T, H]      bf16
+ *   router_logits [T, E]      logits_dtype in {F32, BF16, F16}
+ *   w13           [E, 2I, H]  bf16, rows [0,I) = gate (w1), rows [I,2I) = up (w3)
+ *                             (mixtral_moe.py:64-70,137-143)
+ *   w2            [E, H, I]   bf16 (mixtral_moe.py:75-79)
+ *   out           [T, H]      bf16 (float32 with EM_FLAG_OUT_F32); may alias x
+ *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k), 256-byte aligned
+ * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
+ * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
+ * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.
+ */
+int em_moe_forward(const void* x, const void* router_logits, int logits_dtype,
+                   const void* w13, const void* w2, void* out,
+                   int64_t T, int H, int I, int E, int top_k, int renormalize,
+                   void* workspace, size_t workspace_bytes, unsigned flags,
+                   void* stream);
+
+/*
+ * Byte offsets and element counts of the routing results em_moe_forward leaves
+ * in its workspace, plus the GEMM row-block size it sorts for (the counterpart
+ * of _get_moe_config, fused_moe.py:327-339).  All fields are int64.
+ */
+typedef struct em_moe_layout {
+    int64_t block_size;
+    int64_t topk_weights_off, topk_ids_off;        /* [T*top_k] f32 / i32      */
+    int64_t sorted_ids_off, sorted_len;            /* [sorted_len] i32         */
+    int64_t expert_ids_off, expert_ids_len;        /* [expert_ids_len] i32     */
+    int64_t post_pad_off;                          /* [1] i32                  */
+    int64_t act_off;                               /* [sorted_len, I] bf16     */
+    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 */
+    int64_t total_bytes;
+} em_moe_layout;
+
+int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k,
+                            em_moe_layout* layout);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ELECTROCK_MOE_H */

@@ -1,0 +1,81 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol that
+include/electrock_moe.h declares, and validates arguments before any launch
+(no compute call is made here — there is no GPU in this environment)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from electrock_infer_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "electrock_moe.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(em_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_symbols() == sorted(_lib.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    for name in declared_symbols():
+        assert getattr(lib, name) is not None, name
+    assert lib.em_version() >= 100
+    assert lib.em_error_string(0) == b"success"
+    assert b"workspace" in lib.em_error_string(-5)
+
+
+def test_signatures_carry_no_torch_types():
+    code = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)   # comments cite reference files
+    assert "torch" not in code and "at::" not in code and "#include <hip" not in code
+
+
+def test_argument_errors_are_reported_before_any_launch():
+    lib = _lib.load()
+    # shape errors come first, then null pointers; nothing reaches the device
+    assert lib.em_topk_softmax(None, 0, 4, 128, 2, 1, None, None, None) == -2     # E > 64
+    assert lib.em_topk_softmax(None, 0, 4, 8, 9, 1, None, None, None) == -2       # k > E
+    assert lib.em_topk_softmax(None, 7, 4, 8, 2, 1, None, None, None) == -3       # dtype
+    assert lib.em_topk_softmax(None, 0, 4, 8, 2, 1, None, None, None) == -1       # null
+    assert lib.em_topk_softmax(None, 0, 0, 8, 2, 1, None, None, None) == 0        # empty batch: no-op
+    assert lib.em_moe_align_block_size(None, 0, 16, 8, 0, None, 0, None, 0, None, None) == -2
+    assert lib.em_moe_align_block_size(None, 5, 16, 8, 16, None, 0, None, 0, None, None) == -3
+    assert lib.em_moe_align_block_size(None, 0, 16, 8, 16, None, 136, None, 9, None, None) == -1
+    assert lib.em_silu_and_mul(None, None, 4, 8, 9, None) == -3
+    assert lib.em_silu_and_mul(None, None, 4, 8, 1, None) == -1
+    assert lib.em_silu_and_mul(None, None, 0, 8, 1, None) == 0
+    assert lib.em_moe_sum(None, None, 4, 0, 8, 1, None) == -2
+    assert lib.em_moe_sum(None, None, 4, 2, 8, 1, None) == -1
+    assert lib.em_moe_forward(None, None, 1, None, None, None, 4, 4097, 512, 8, 2, 1, None, 0, 0, None) == -2
+    assert lib.em_moe_forward(None, None, 1, None, None, None, 4, 4096, 512, 8, 2, 1, None, 0, 0, None) == -1
+
+
+def test_workspace_layout_is_consistent():
+    lib = _lib.load()
+    for T, H, I in [(1, 4096, 14336), (64, 4096, 14336), (256, 4096, 14336), (8192, 4096, 14336),
+                    (64, 256, 512), (4096, 6144, 16384)]:
+        L = _lib.workspace_layout(T, H, I, 8, 2)
+        assert lib.em_moe_workspace_bytes(T, H, I, 8, 2) == L.total_bytes
+        assert L.block_size in (16, 64)
+        assert L.sorted_len % L.block_size == 0 and L.sorted_len >= T * 2 + 8 * (L.block_size - 1)
+        assert L.expert_ids_len * L.block_size == L.sorted_len
+        offs = [L.topk_weights_off, L.topk_ids_off, L.sorted_ids_off, L.expert_ids_off, L.post_pad_off,
+                L.act_off, L.y_off, L.total_bytes]
+        assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
+        assert L.y_off - L.act_off >= L.sorted_len * I * 2
+        assert L.total_bytes - L.y_off >= L.ksplit * T * 2 * H * 4
+    assert lib.em_moe_workspace_bytes(4, 4097, 512, 8, 2) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()
