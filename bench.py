@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the Mixtral-8x7B MoE layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T] [--no-cpu] [--no-table]
+
+A "step" is one call of the layer (router, expert sort, w13 GEMM + SiLU*mul,
+w2 GEMM, top-k combine) on one batch of T tokens resident in HBM.  The headline
+workload is the decode batch T=64 of the 8x7B shape (H=4096, I=14336, E=8,
+top-2 renormalised, bf16, N(0,1) router logits); `value` is T / (time per step).
+
+One JSON line is printed.  Besides the contract fields it carries
+  roofline      the dominant kernel (w13 GEMM + SiLU*mul), timed alone with HIP
+                events on the stream it is launched on, against 8 TB/s of HBM
+  cpu_baseline  the reference-style torch CPU expert loop (oracle port) timed on
+                the host cores on the same workload
+  table         layer latency / HBM GB/s / MFMA TFLOP/s for the other batch sizes
+                of the decode list and the T=8192 prefill case
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+H, I, E, TOPK = 4096, 14336, 8, 2
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tokens", type=int, default=64, help="batch size T of the headline workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
+    return ap.parse_args()
+
+
+def make_weights(torch, dev):
+    g = torch.Generator(device=dev).manual_seed(0)
+    w13 = torch.empty(E, 2 * I, H, device=dev, dtype=torch.bfloat16)
+    w2 = torch.empty(E, H, I, device=dev, dtype=torch.bfloat16)
+    for e in range(E):
+        w13[e] = (torch.randn(2 * I, H, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+        w2[e] = (torch.randn(H, I, generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    return w13, w2
+
+
+def make_batch(torch, dev, T, seed=0, logits="normal"):
+    g = torch.Generator(device=dev).manual_seed(1000 + seed)
+    x = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    lg = torch.randn(T, E, generator=g, device=dev, dtype=torch.float32)
+    if logits == "zipf":
+        ranks = torch.arange(1, E + 1, dtype=torch.float32) ** -1.2
+        perm = torch.randperm(E, generator=torch.Generator().manual_seed(seed))
+        lg = lg + torch.log(ranks / ranks.sum())[perm].to(dev)
+    elif logits == "two_experts":
+        lg[:, :2] += 20.0
+    return x, lg.to(torch.bfloat16)
+
+
+class LayerRunner:
+    """Calls em_moe_forward through the C ABI with pre-allocated buffers."""
+
+    def __init__(self, torch, T, w13, w2, x, lg):
+        import ctypes
+        from electrock_infer_amd import _lib
+        from electrock_infer_amd.layers.moe.fused_moe import MoeWorkspace
+        self.torch, self._lib, self.ctypes = torch, _lib, ctypes
+        self.T, self.w13, self.w2, self.x, self.lg = T, w13, w2, x, lg
+        self.ws = MoeWorkspace(x.device, T, H, I, E, TOPK)
+        self.out = torch.empty_like(x)
+        self.lib = _lib.load()
+
+    def __call__(self, flags=0):
+        code = self.lib.em_moe_forward(
+            self.x.data_ptr(), self.lg.data_ptr(), self._lib.DTYPE_BF16, self.w13.data_ptr(), self.w2.data_ptr(),
+            self.out.data_ptr(), self.T, H, I, E, TOPK, 1, self.ws.buffer.data_ptr(),
+            self.ctypes.c_size_t(self.ws.buffer.numel()), flags,
+            self.torch.cuda.current_stream().cuda_stream)
+        self._lib.check(code, "em_moe_forward")
+
+    def n_active(self):
+        return int(self.ws.topk_ids().unique().numel())
+
+
+def time_calls(torch, fn, steps, warmup):
+    """Average milliseconds per call: HIP events on the current stream around `steps` calls."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall_ms
+
+
+def layer_bytes(T, n_active):
+    """Algorithmic HBM bytes of one layer call: active expert weights once, x in, out, logits."""
+    return n_active * 3 * H * I * 2 + 2 * T * H * 2 + T * E * 2
+
+
+def layer_flops(T):
+    return T * TOPK * 6 * H * I
+
+
+def measure(torch, T, w13, w2, steps, warmup, logits="normal"):
+    from electrock_infer_amd import _lib
+    x, lg = make_batch(torch, w13.device, T, logits=logits)
+    run = LayerRunner(torch, T, w13, w2, x, lg)
+    run()
+    torch.cuda.synchronize()
+    na = run.n_active()
+    ms, wall_ms = time_calls(torch, run, steps, warmup)
+    only = lambda keep: (_lib.FLAG_SKIP_ROUTER | _lib.FLAG_SKIP_ALIGN | _lib.FLAG_SKIP_GEMM1 |
+                         _lib.FLAG_SKIP_GEMM2 | _lib.FLAG_SKIP_COMBINE) & ~keep
+    stage = {}
+    for name, flag in (("gemm1", _lib.FLAG_SKIP_GEMM1), ("gemm2", _lib.FLAG_SKIP_GEMM2),
+                       ("router", _lib.FLAG_SKIP_ROUTER), ("align", _lib.FLAG_SKIP_ALIGN),
+                       ("combine", _lib.FLAG_SKIP_COMBINE)):
+        stage[name] = time_calls(torch, lambda f=only(flag): run(f), steps, max(2, warmup // 4))[0]
+    return {"T": T, "logits": logits, "ms": ms, "wall_ms": wall_ms, "n_active": na, "stage_ms": stage,
+            "tokens_per_s": T / ms * 1e3, "hbm_gbs": layer_bytes(T, na) / ms / 1e6,
+            "tflops": layer_flops(T) / ms / 1e9}
+
+
+def cpu_baseline(torch, T, w13, w2):
+    """Reference-style torch CPU expert loop (oracle port) on the same workload, host cores."""
+    from oracle import moe_oracle as O
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
+    torch.set_num_threads(cores)
+    x, lg = make_batch(torch, w13.device, T)
+    xc, lc = x.float().cpu(), lg.float().cpu()
+    w13c, w2c = w13.cpu().float(), w2.cpu().float()      # the CPU path holds fp32 weights
+    O.moe_layer_fp32(xc, lc, w13c, w2c)                  # warm-up
+    iters, t0 = 0, time.perf_counter()
+    while iters < 3 or (time.perf_counter() - t0 < 10.0 and iters < 200):
+        O.moe_layer_fp32(xc, lc, w13c, w2c)
+        iters += 1
+    sec = (time.perf_counter() - t0) / iters
+    return {"value": T / sec, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{iters} calls of the fp32 torch expert loop (oracle.moe_layer_fp32) on the same "
+                      f"T={T} 8x7B batch, weights pre-cast to fp32, {sec * 1e3:.1f} ms per call"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: all experts are resident on a single MI355X and the layer uses "
+              "no collectives; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from electrock_infer_amd import _lib
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w13, w2 = make_weights(torch, dev)
+
+    T = args.tokens
+    head = measure(torch, T, w13, w2, args.steps, args.warmup)
+    g1_ms = head["stage_ms"]["gemm1"]
+    g1_bytes = head["n_active"] * 2 * I * H * 2 + T * H * 2   # w13 of the active experts + x
+    roofline = {"kernel": "w13 GEMM + SiLU*mul", "bound": "hbm", "achieved": g1_bytes / g1_ms / 1e6,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": None,
+                "bytes_per_launch": g1_bytes, "avg_launch_ms": g1_ms}
+    roofline["frac"] = roofline["achieved"] / roofline["peak"]
+
+    table = []
+    if not args.no_table:
+        for t in (1, 8, 32, 256):
+            if t != T:
+                table.append(measure(torch, t, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2)))
+        for lgk in ("normal", "zipf", "two_experts"):
+            r = measure(torch, 8192, w13, w2, 10, 3, logits=lgk)
+            r["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
+            table.append(r)
+    for r in [head] + table:
+        r["hbm_frac"] = r["hbm_gbs"] / HBM_PEAK_GBS
+
+    result = {
+        "metric": "Mixtral-8x7B MoE layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"Mixtral-8x7B MoE layer decode T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
+                               f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
+                   "tokens": T, "n_active_experts": head["n_active"]},
+        "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(torch, T, w13, w2),
+        "table": table,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

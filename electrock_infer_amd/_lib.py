@@ -33,7 +33,7 @@ class MoeLayout(ctypes.Structure):
     """Mirror of struct em_moe_layout."""
     _fields_ = [(n, ctypes.c_int64) for n in (
         "block_size", "topk_weights_off", "topk_ids_off", "sorted_ids_off", "sorted_len",
-        "expert_ids_off", "expert_ids_len", "post_pad_off", "act_off", "y_off", "ksplit",
+        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "act_off", "y_off", "ksplit",
         "total_bytes")]
 
 

@@ -26,7 +26,7 @@ template <typename IdT>
 __global__ __launch_bounds__(kAlignThreads) void align_kernel(
     const IdT* __restrict__ ids, int64_t numel, int E, int block,
     int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
-    int64_t eid_len, int32_t* __restrict__ post_pad) {
+    int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out) {
     __shared__ int32_t hist[kAlignWaves][kMaxExperts];  // pass 1 counts, then write bases
     __shared__ int32_t seg_begin[kMaxExperts + 1];      // padded exclusive prefix
 
@@ -79,6 +79,7 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
         post_pad[0] = run;
     }
     __syncthreads();  // also orders the -1 / 0 fill before the scatter below
+    if (seg_out != nullptr && tid <= E) seg_out[tid] = seg_begin[tid];  // padded start of every expert segment
 
     // block -> expert table
     if (tid < E) {
@@ -107,14 +108,14 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
 
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
-                 int32_t* post_pad, hipStream_t s) {
+                 int32_t* post_pad, int32_t* seg_out, hipStream_t s) {
     const dim3 grid(1), blk(kAlignThreads);
     if (itype == EM_ITYPE_I32) {
         hipLaunchKernelGGL(align_kernel<int32_t>, grid, blk, 0, s, static_cast<const int32_t*>(ids),
-                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad);
+                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else if (itype == EM_ITYPE_I64) {
         hipLaunchKernelGGL(align_kernel<int64_t>, grid, blk, 0, s, static_cast<const int64_t*>(ids),
-                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad);
+                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else {
         return EM_ERR_BAD_DTYPE;
     }

@@ -12,14 +12,27 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 inline bool dtype_ok(int d) { return d == EM_DTYPE_F32 || d == EM_DTYPE_BF16 || d == EM_DTYPE_F16; }
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// Up to this many tokens the weight-streaming GEMM runs (16-row sorted blocks, a
+// couple of MFMA fragments per expert); above it the tiled kernels take over.
+constexpr int64_t kStreamMaxT = 64;
+
 // Counterpart of _get_moe_config (fused_moe.py:327-339): rows per sorted block.
 // An expert receives at most T rows, so up to 16 tokens one 16-row MFMA
-// fragment per expert always suffices; above that one 64-row block per expert
-// keeps each weight tile read by a single workgroup for decode batches.
-inline int choose_block(int64_t T) { return T <= 16 ? 16 : 64; }
+// fragment per expert always suffices.
+inline int choose_block(int64_t T) { return T <= kStreamMaxT ? 16 : 64; }
 // Split of the w2 reduction (K = I) across workgroups for small batches, where
 // (row blocks) x (H / 128 column tiles) alone would leave most CUs idle.
-inline int choose_ksplit(int64_t T) { return T <= 64 ? 8 : (T <= 512 ? 4 : 1); }
+inline int choose_ksplit(int64_t T, int I) {
+    if (T > kStreamMaxT) return T <= 512 ? 4 : 1;
+    // Streaming kernel: (active experts) x (H / 64) row tiles should give every CU
+    // work.  From ~17 tokens on all eight experts are almost surely active and one
+    // K slice per tile measures fastest; below that the reduction is split four ways.
+    // The kernel needs I / ksplit to be a multiple of 256.
+    const int want = T <= 16 ? 4 : 1;
+    for (int ks = want; ks >= 1; --ks)
+        if (I % (ks * 256) == 0) return ks;
+    return want;
+}
 
 bool shapes_ok(int64_t T, int H, int I, int E, int top_k) {
     return T >= 0 && H > 0 && I > 0 && E >= 1 && E <= kMaxExperts && top_k >= 1 && top_k <= kMaxTopK &&
@@ -67,7 +80,7 @@ int em_moe_align_block_size(const void* topk_ids, int ids_itype, int64_t numel, 
         return EM_ERR_NULL_POINTER;
     if (sorted_len < 0 || expert_ids_len < 0) return EM_ERR_BUFFER_SIZE;
     return launch_align(topk_ids, ids_itype, numel, num_experts, block_size, sorted_token_ids, sorted_len,
-                        expert_ids, expert_ids_len, num_tokens_post_pad, as_stream(stream));
+                        expert_ids, expert_ids_len, num_tokens_post_pad, nullptr, as_stream(stream));
 }
 
 int em_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, void* stream) {
@@ -106,8 +119,9 @@ int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_la
     L->expert_ids_len = sorted_len / block;
     L->expert_ids_off = take(L->expert_ids_len * 4);
     L->post_pad_off = take(4);
+    L->seg_begin_off = take((E + 1) * 4);
     L->act_off = take(sorted_len * static_cast<int64_t>(I) * 2);
-    L->ksplit = choose_ksplit(T);
+    L->ksplit = choose_ksplit(T, I);
     L->y_off = take(L->ksplit * slots * static_cast<int64_t>(H) * 4);
     L->total_bytes = off;
     return 0;
@@ -145,6 +159,7 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
     int32_t* eids = reinterpret_cast<int32_t*>(ws + L.expert_ids_off);
     int32_t* post_pad = reinterpret_cast<int32_t*>(ws + L.post_pad_off);
+    int32_t* seg_begin = reinterpret_cast<int32_t*>(ws + L.seg_begin_off);
     float* topk_w = reinterpret_cast<float*>(ws + L.topk_weights_off);
     int32_t* topk_ids = reinterpret_cast<int32_t*>(ws + L.topk_ids_off);
     p.sorted_ids = sorted;
@@ -166,15 +181,16 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
     }
     if (!(flags & EM_FLAG_SKIP_ALIGN)) {
         rc = launch_align(topk_ids, EM_ITYPE_I32, T * top_k, E, p.block, sorted, L.sorted_len, eids,
-                          L.expert_ids_len, post_pad, s);
+                          L.expert_ids_len, post_pad, seg_begin, s);
         if (rc != 0) return rc;
     }
+    const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
-        rc = launch_gemm_generic(p, 1, s);
+        rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s) : launch_gemm_generic(p, 1, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
-        rc = launch_gemm_generic(p, 2, s);
+        rc = use_stream ? launch_gemm_stream(p, seg_begin, 2, s) : launch_gemm_generic(p, 2, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_COMBINE)) {

@@ -73,7 +73,8 @@ int launch_router(const void* logits, int logits_dtype, int64_t T, int E, int k,
                   float* w, int32_t* ids, hipStream_t s);
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
-                 int32_t* post_pad, hipStream_t s);
+                 int32_t* post_pad, int32_t* seg_out /* [E+1] padded segment starts, may be null */,
+                 hipStream_t s);
 int launch_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, hipStream_t s);
 int launch_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype, hipStream_t s);
 
@@ -95,6 +96,8 @@ struct MoeProblem {
     int ksplit;
 };
 int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s);  // mode 1: w13+SiLU*mul, 2: w2
+bool stream_supported(const MoeProblem& p);
+int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s);
 int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s);
 
 }  // namespace em

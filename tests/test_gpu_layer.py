@@ -9,7 +9,9 @@ fp32 result to bf16 alone costs about 1.4e-3 mean relative error and up to
 half a bf16 ulp (0.0156 for |v| in [4, 8), 0.031 for [8, 16)) — so every case
 reports the measured errors of the fp32 output and of the bf16 output, and
 asserts
-    fp32 output : mean_rel <= TOL_MEAN_REL_F32, max_abs <= TOL_MAX_ABS_F32
+    fp32 output : mean_rel <= TOL_MEAN_REL_F32, max_abs <= TOL_MAX_ABS_F32 * max|ref|
+                  (the activation rounding is a relative error, so the bound scales
+                  with the output magnitude: max|ref| is ~9 at 8x7B and ~16 at 8x22B)
     bf16 output : equal to the rounded fp32 output within 1 bf16 ulp, and
                   mean_rel <= TOL_MEAN_REL_BF16
 """
@@ -20,7 +22,7 @@ import numpy as np
 import pytest
 import torch
 
-from electrock_infer_amd import FusedMoE, fused_experts
+from electrock_infer_amd import FusedMoE, fused_experts, moe_align_block_size
 from electrock_infer_amd.layers.moe.fused_moe import get_workspace
 from oracle import c_oracle, moe_oracle as O
 from tests.gpu_util import DEV, announce, error_stats, gpu_inputs, oracle_rows
@@ -28,7 +30,7 @@ from tests.gpu_util import DEV, announce, error_stats, gpu_inputs, oracle_rows
 pytestmark = pytest.mark.gpu
 
 TOL_MEAN_REL_F32 = 2.5e-3    # one bf16 rounding of the SiLU*mul activations feeds the w2 MFMA
-TOL_MAX_ABS_F32 = 2e-2
+TOL_MAX_ABS_F32 = 4e-3       # times max|ref|
 TOL_MEAN_REL_BF16 = 3.5e-3   # + the final rounding of the output to bf16
 
 REPORT = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out", "layer_errors.jsonl")
@@ -61,7 +63,7 @@ def check_outputs(case, out_f32, out_bf16, ref):
     f = error_stats(out_f32, ref)
     b = error_stats(out_bf16.float(), ref)
     record(case, f32=f, bf16=b, ref_absmean=float(ref.abs().mean()), ref_absmax=float(ref.abs().max()))
-    assert f["mean_rel"] <= TOL_MEAN_REL_F32 and f["max_abs"] <= TOL_MAX_ABS_F32, (case, f)
+    assert f["mean_rel"] <= TOL_MEAN_REL_F32 and f["max_abs"] <= TOL_MAX_ABS_F32 * float(ref.abs().max()), (case, f)
     assert b["mean_rel"] <= TOL_MEAN_REL_BF16, (case, b)
     rounded = out_f32.to(torch.bfloat16).float()
     ulp = torch.maximum(rounded.abs(), torch.tensor(1e-30, device=rounded.device)) * 2.0 ** -7
@@ -99,18 +101,19 @@ def test_layer_golden_fixture_c1():
     ws = get_workspace(DEV, 64, 256, 512, 8, 2)
     assert np.array_equal(ws.topk_ids().cpu().numpy(), gold["topk_ids"])
     np.testing.assert_allclose(ws.topk_weights().cpu().numpy(), gold["topk_weights"], rtol=4e-6)
-    assert ws.block_size == 64
-    n = gold["sorted_token_ids"].size
-    assert np.array_equal(ws.sorted_token_ids().cpu().numpy()[:n], gold["sorted_token_ids"])
-    assert np.array_equal(ws.expert_ids().cpu().numpy(), gold["expert_ids"])
-    assert np.array_equal(ws.num_tokens_post_pad().cpu().numpy(), gold["num_tokens_post_pad"])
+    # the fixture's sort uses the reference's block size for T=64 (64 rows); the fused
+    # path sorts for its own tile, so the op is run on the layer's topk_ids
+    s_ids, e_ids, n_pad = moe_align_block_size(ws.topk_ids(), 64, 8)
+    assert np.array_equal(s_ids.cpu().numpy(), gold["sorted_token_ids"])
+    assert np.array_equal(e_ids.cpu().numpy(), gold["expert_ids"])
+    assert np.array_equal(n_pad.cpu().numpy(), gold["num_tokens_post_pad"])
     # fp32-input fixture vs bf16-input GPU run: input rounding dominates (about 4e-3 relative)
     st = error_stats(out.cpu(), torch.from_numpy(gold["out"]))
     record("golden_c1", f32=st)
     assert st["mean_rel"] < 1e-2
     ref = O.moe_layer_fp32(xb, lg, w13b, w2b)
     st = error_stats(out.cpu(), ref)
-    assert st["mean_rel"] <= TOL_MEAN_REL_F32 and st["max_abs"] <= TOL_MAX_ABS_F32
+    assert st["mean_rel"] <= TOL_MEAN_REL_F32 and st["max_abs"] <= TOL_MAX_ABS_F32 * float(ref.abs().max())
 
 
 @pytest.fixture(scope="module")

@@ -162,10 +162,12 @@ def test_silu_and_mul(dtype, rows, d):
         assert torch.allclose(got, ref, rtol=1e-6, atol=1e-7)
     else:
         # the device exp may differ from the CPU's in the last ulp, which can move the
-        # intermediate rounding by one unit: allow 1 ulp of the 16-bit type, and most exact
-        ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+        # intermediate rounding by one unit and then the product's: allow 2 ulp of the
+        # 16-bit type, with nearly all elements exact
+        ulp = 2.0 ** -6 if dtype == torch.bfloat16 else 2.0 ** -9
         d_ = (got.float() - ref.float()).abs()
-        assert (d_ <= ulp * ref.float().abs() + 1e-30).all()
+        floor = 6.2e-8 if dtype == torch.float16 else 1e-30      # fp16 results can be subnormal
+        assert (d_ <= ulp * ref.float().abs() + floor).all()
         assert (d_ == 0).float().mean() > 0.98
     # the reference's own check (test/example/test_silu.py:16-27)
     lib = torch.nn.functional.silu(x[:, :d].float()) * x[:, d:].float()
@@ -181,7 +183,8 @@ def test_moe_sum(dtype, T, H):
     out = torch.full((T, H), 99.0, dtype=dtype, device=DEV)
     assert _C.moe_sum(x.to(DEV), out) is None
     assert torch.equal(out.cpu(), O.moe_sum(x))               # one rounding of an exact sum: bit-exact
-    assert torch.allclose(out.cpu().float(), torch.sum(x.float(), 1), atol=1e-2)  # test_moe_sum.py:70-76
+    # the reference's own check is fp16 with atol 1e-2 (test_moe_sum.py:70-76); half a bf16 ulp near 8 is 3.1e-2
+    assert torch.allclose(out.cpu().float(), torch.sum(x.float(), 1), atol=3.2e-2 if dtype == torch.bfloat16 else 1e-2)
     with pytest.raises(RuntimeError, match="top_k=2"):
         _C.moe_sum(torch.zeros(4, 3, 8, device=DEV, dtype=dtype), torch.zeros(4, 8, device=DEV, dtype=dtype))
 
