@@ -19,7 +19,10 @@ constexpr int64_t kStreamMaxT = 64;
 // Counterpart of _get_moe_config (fused_moe.py:327-339): rows per sorted block.
 // An expert receives at most T rows, so up to 16 tokens one 16-row MFMA
 // fragment per expert always suffices.
-inline int choose_block(int64_t T) { return T <= kStreamMaxT ? 16 : 64; }
+// From this many tokens on (>= 256 rows per expert on average for 8 experts, top-2)
+// the 256 x 256 tiled kernel runs and the sort pads experts to 256 rows.
+constexpr int64_t kTileMinT = 1024;
+inline int choose_block(int64_t T) { return T <= kStreamMaxT ? 16 : (T < kTileMinT ? 64 : 256); }
 // Split of the w2 reduction (K = I) across workgroups for small batches, where
 // (row blocks) x (H / 128 column tiles) alone would leave most CUs idle.
 inline int choose_ksplit(int64_t T, int I) {
@@ -185,12 +188,15 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
         if (rc != 0) return rc;
     }
     const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
+    const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T >= kTileMinT && tile_supported(p);
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
-        rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s) : launch_gemm_generic(p, 1, s);
+        rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s)
+             : use_tile ? launch_gemm_tile(p, 1, s) : launch_gemm_generic(p, 1, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
-        rc = use_stream ? launch_gemm_stream(p, seg_begin, 2, s) : launch_gemm_generic(p, 2, s);
+        rc = use_stream ? launch_gemm_stream(p, seg_begin, 2, s)
+             : use_tile ? launch_gemm_tile(p, 2, s) : launch_gemm_generic(p, 2, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_COMBINE)) {

@@ -211,8 +211,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 }  // namespace
 
 int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s) {
-    if (p.block != 16 && p.block != 64) return EM_ERR_UNSUPPORTED;
-    const unsigned mblocks = static_cast<unsigned>(p.sorted_len / p.block);
+    if (p.block != 16 && p.block % 64 != 0) return EM_ERR_UNSUPPORTED;  // one 64-row tile never spans experts
+    const int tile_rows = (p.block == 16) ? 16 : 64;
+    const unsigned mblocks = static_cast<unsigned>(p.sorted_len / tile_rows);
     if (mblocks == 0) return 0;
     const dim3 blk(kThreads);
     if (mode == 1) {
