@@ -2,15 +2,21 @@
 // where the layer is bound by the bf16 MFMA rate.
 //
 //   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile 256 sorted rows x 256
-//              weight rows, K in steps of 64 through a double-buffered LDS tile
-//              (2 x 72 KB with the 144-byte row pitch that keeps b128 reads
-//              conflict-free)
+//              weight rows; K in steps of 32 through a ring of four 32 KB LDS stages
+//   loads      global -> LDS directly (global_load_lds_dwordx4), no registers in
+//              between, so three stages (96 KB per CU) are in flight while the
+//              fourth is multiplied; completion is tracked by hand with
+//              s_waitcnt vmcnt + one s_barrier per stage
+//   LDS        rows are 64 B; the 16-byte pieces of every 4-row group are XOR-
+//              swizzled so that the 16 lanes of a b128 operand read hit 16 banks groups
 //   wave       128 x 64 sub-tile = 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators
 //   MODE 1     the wave's two N fragments are 32 gate rows j and the matching 32
 //              up rows I + j, so SiLU(g) * u is lane-local in the epilogue
 //   MODE 2     256 rows of w2[e]; fp32 partial rows are scattered to y[slot]
 //   rows       A rows are gathered through sorted_token_ids (MODE 1) or read in
-//              sorted order from act (MODE 2); the sort pads every expert to 256
+//              sorted order from act (MODE 2); the sort pads every expert to 256.
+//              Pad rows read token 0: their products only reach pad rows of act,
+//              which no output row depends on.
 //   order      workgroup ids are dealt to the 8 XCDs round-robin by the hardware;
 //              they are re-mapped so that each XCD walks one contiguous range of
 //              tiles, ordered 4 row blocks x all column tiles, which lets the 32
@@ -20,15 +26,33 @@
 namespace em {
 namespace {
 
-constexpr int kTM = 256, kTN = 256, kTK = 64;
+constexpr int kTM = 256, kTN = 256, kTK = 32;
 constexpr int kThreads = 512;
-constexpr int kPitch = kTK * 2 + 16;                 // 144 B
-constexpr int kStageBytes = (kTM + kTN) * kPitch;    // 73,728 B
-constexpr int kLdsBytes = 2 * kStageBytes;           // 147,456 B
+constexpr int kStages = 4;
+constexpr int kRegionBytes = kTM * kTK * 2;          // 16 KB: A rows, then 16 KB of B rows
+constexpr int kStageBytes = 2 * kRegionBytes;        // 32 KB
+constexpr int kLdsBytes = kStages * kStageBytes;     // 128 KB
 constexpr int kGroupM = 4;
 constexpr int kXcds = 8;
+constexpr int kDmaPerStage = kStageBytes / (kThreads * 16);  // 4 per thread
 
-__device__ __forceinline__ u32x4_t ld16(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+// M0 is a reserved register that the compiler never keeps live values in here (the
+// kernel has no dynamically indexed register arrays); naming it as a clobber documents
+// the write and only triggers an advisory warning.
+#pragma clang diagnostic ignored "-Winline-asm"
+
+// One wave copies 64 x 16 B from per-lane global addresses to 1 KB of LDS starting at
+// the wave-uniform byte address `lds_addr`.  The compiler does not see the LDS write:
+// every consumer sits behind wait_dma<>() + block_barrier().
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_dma() {  // at most N of this wave's copies still in flight
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+__device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 template <int MODE>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, int ntiles_n) {
@@ -58,43 +82,42 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
     const int expert = p.expert_ids[m0 / p.block];
     const int K = (MODE == 1) ? p.H : p.I;
 
-    // ---- per-thread global sources: chunk c = tid + i*512 -> row c/8, 16-byte piece c%8 ----
-    const int lrow = tid >> 3;
-    const int lkc = (tid & 7) * 8;
-    const uint16_t* a_src[4];
-    const uint16_t* b_src[4];
+    // ---- copy plan: copy n of a stage lands at region (n >> 1), byte (n & 1) * 8 KB + wave * 1 KB + lane * 16.
+    // Byte o of a region holds piece q ^ (u & 3) of 4-row group u = o / 256, q = (row & 3) * 4 + piece.
+    const uint16_t* src[kDmaPerStage];
     const uint16_t* wbase = (MODE == 1) ? p.w13 + static_cast<int64_t>(expert) * 2 * p.I * p.H
                                         : p.w2 + static_cast<int64_t>(expert) * p.H * p.I;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = lrow + i * 64;
-        if (MODE == 1) {
-            const int slot = p.sorted_ids[m0 + r];
-            a_src[i] = (slot >= 0) ? p.x + static_cast<int64_t>(slot / p.top_k) * p.H + lkc : nullptr;
-            // LDS row r of the B tile: wave column r/64, gate (0) or up (1) half, j offset r%32
-            const int64_t grow = static_cast<int64_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31);
-            b_src[i] = wbase + grow * K + lkc;
+    for (int n = 0; n < kDmaPerStage; ++n) {
+        const int o = (n & 1) * 8192 + wave * 1024 + lane * 16;
+        const int u = o >> 8;
+        const int q = ((o >> 4) & 15) ^ (u & 3);
+        const int r = u * 4 + (q >> 2);
+        const int piece = q & 3;
+        if ((n >> 1) == 0) {
+            if (MODE == 1) {
+                const int slot = p.sorted_ids[m0 + r];
+                const int tok = (slot >= 0) ? slot / p.top_k : 0;
+                src[n] = p.x + static_cast<int64_t>(tok) * p.H + piece * 8;
+            } else {
+                src[n] = p.act + (m0 + r) * static_cast<int64_t>(p.I) + piece * 8;
+            }
         } else {
-            a_src[i] = p.act + (m0 + r) * static_cast<int64_t>(p.I) + lkc;
-            b_src[i] = wbase + static_cast<int64_t>(nt * kTN + r) * K + lkc;
+            int64_t grow;
+            if (MODE == 1)  // LDS row r of the B tile: wave column r/64, gate (0) or up (1) half, j offset r%32
+                grow = static_cast<int64_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31);
+            else
+                grow = static_cast<int64_t>(nt) * kTN + r;
+            src[n] = wbase + grow * K + piece * 8;
         }
     }
-
-    u32x4_t a_reg[4], b_reg[4];
-    auto load_global = [&](int k0) {
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
+    const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+    auto issue = [&](int stage_k, int buf) {  // stage_k: K step index, buf: ring slot
+        const int k0 = stage_k * kTK;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a_reg[i] = (a_src[i] != nullptr) ? ld16(a_src[i] + k0) : u32x4_t{0, 0, 0, 0};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) b_reg[i] = ld16(b_src[i] + k0);
-    };
-    auto store_lds = [&](int buf) {
-        uint8_t* sa = smem + buf * kStageBytes;
-        uint8_t* sb = sa + kTM * kPitch;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4_t*>(sa + (lrow + i * 64) * kPitch + lkc * 2) = a_reg[i];
-            *reinterpret_cast<u32x4_t*>(sb + (lrow + i * 64) * kPitch + lkc * 2) = b_reg[i];
-        }
+        for (int n = 0; n < kDmaPerStage; ++n)
+            dma16(src[n] + k0, dma_base + buf * kStageBytes + (n >> 1) * kRegionBytes + (n & 1) * 8192);
     };
 
     f32x16_t acc[4][2];
@@ -105,36 +128,44 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
 
+    // ---- operand reads: lane (r32, kh) takes row r32 of a 32-row fragment, piece ks*2 + kh ----
     const int r32 = lane & 31;
-    const int kh = lane >> 5;  // which 8-element half of a 16-wide K step
-    const int a_off = (wm * 128 + r32) * kPitch + kh * 16;
-    const int b_off = kTM * kPitch + (wn * 64 + r32) * kPitch + kh * 16;
+    const int kh = lane >> 5;
+    const int sw = (r32 >> 2) & 3;  // (row / 4) & 3 is the same for every fragment of this lane
+    int a_off[2], b_off[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int piece = (ks * 2 + kh) ^ sw;
+        const int ra = wm * 128 + r32, rb = wn * 64 + r32;
+        a_off[ks] = (ra >> 2) * 256 + ((ra & 3) * 4 + piece) * 16;
+        b_off[ks] = kRegionBytes + (rb >> 2) * 256 + ((rb & 3) * 4 + piece) * 16;
+    }
 
     const int nk = K / kTK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * kTK);
-        const uint8_t* s = smem + buf * kStageBytes;
 #pragma unroll
-        for (int ks = 0; ks < kTK / 16; ++ks) {
+    for (int st = 0; st < kStages - 1; ++st)
+        if (st < nk) issue(st, st);
+    for (int kt = 0; kt < nk; ++kt) {
+        // stage kt has landed once at most the copies of the (up to two) younger stages are in flight
+        if (kt + 2 < nk) wait_dma<2 * kDmaPerStage>();
+        else if (kt + 1 < nk) wait_dma<kDmaPerStage>();
+        else wait_dma<0>();
+        block_barrier();  // everyone's part of stage kt is in LDS; everyone is done reading stage kt-1
+        if (kt + kStages - 1 < nk) issue(kt + kStages - 1, (kt + kStages - 1) % kStages);
+        const uint8_t* s = smem + (kt % kStages) * kStageBytes;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
             bf16x8_t af[4], bfr[2];
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
-                af[mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off + mi * 32 * kPitch + ks * 32);
+            for (int mi = 0; mi < 4; ++mi) af[mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off[ks] + mi * 2048);
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-                bfr[ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off + ni * 32 * kPitch + ks * 32);
+            for (int ni = 0; ni < 2; ++ni) bfr[ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off[ks] + ni * 2048);
 #pragma unroll
             for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < 2; ++ni)
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0);
         }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
-        __syncthreads();
     }
 
     // ---- epilogue: element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
@@ -169,7 +200,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
 
 bool tile_supported(const MoeProblem& p) {
     return p.block == kTM && p.ksplit == 1 && p.H % kTN == 0 && p.I % 128 == 0 && p.H % kTK == 0 &&
-           p.I % kTK == 0;
+           p.I % kTK == 0 && p.T > 0;
 }
 
 int launch_gemm_tile(const MoeProblem& p, int mode, hipStream_t s) {
