@@ -2,14 +2,18 @@
 // where the layer is bound by the bf16 MFMA rate.
 //
 //   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile 256 sorted rows x 256
-//              weight rows; K in steps of 32 through a ring of four 32 KB LDS stages
+//              weight rows; K in steps of 64 through two 64 KB LDS stages
 //   loads      global -> LDS directly (global_load_lds_dwordx4), no registers in
-//              between, so three stages (96 KB per CU) are in flight while the
-//              fourth is multiplied; completion is tracked by hand with
-//              s_waitcnt vmcnt + one s_barrier per stage
-//   LDS        rows are 64 B; the 16-byte pieces of every 4-row group are XOR-
-//              swizzled so that the 16 lanes of a b128 operand read hit 16 banks groups
-//   wave       128 x 64 sub-tile = 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators
+//              between; eight lanes fetch one full 128-byte line of a row (measured
+//              L2 -> CU feed: ~23 TB/s with 128 B per row against ~16 TB/s with 64 B);
+//              the copy of stage k+1 runs while stage k is multiplied; completion is
+//              tracked by hand with s_waitcnt vmcnt + one s_barrier per stage
+//   LDS        rows are 128 B; the 16-byte pieces of every 2-row group are XOR-
+//              swizzled so that the 16 lanes of a b128 operand read hit 16 bank groups
+//   wave       128 x 64 sub-tile = 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (the
+//              16x16x32 form runs at half this rate on gfx950); operand fragments are
+//              double-buffered in registers and their LDS reads are woven between the
+//              MFMAs of the previous 16-wide K step, also across the stage barrier
 //   MODE 1     the wave's two N fragments are 32 gate rows j and the matching 32
 //              up rows I + j, so SiLU(g) * u is lane-local in the epilogue
 //   MODE 2     256 rows of w2[e]; fp32 partial rows are scattered to y[slot]
@@ -26,15 +30,16 @@
 namespace em {
 namespace {
 
-constexpr int kTM = 256, kTN = 256, kTK = 32;
+constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kThreads = 512;
-constexpr int kStages = 4;
-constexpr int kRegionBytes = kTM * kTK * 2;          // 16 KB: A rows, then 16 KB of B rows
-constexpr int kStageBytes = 2 * kRegionBytes;        // 32 KB
+constexpr int kStages = 2;
+constexpr int kRegionBytes = kTM * kTK * 2;          // 32 KB: A rows, then 32 KB of B rows
+constexpr int kStageBytes = 2 * kRegionBytes;        // 64 KB
 constexpr int kLdsBytes = kStages * kStageBytes;     // 128 KB
 constexpr int kGroupM = 4;
 constexpr int kXcds = 8;
-constexpr int kDmaPerStage = kStageBytes / (kThreads * 16);  // 4 per thread
+constexpr int kDmaPerStage = kStageBytes / (kThreads * 16);  // 8 per thread
+constexpr int kDmaHalf = kDmaPerStage / 2;                   // first half A rows, second half B rows
 
 // M0 is a reserved register that the compiler never keeps live values in here (the
 // kernel has no dynamically indexed register arrays); naming it as a clobber documents
@@ -82,19 +87,19 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
     const int expert = p.expert_ids[m0 / p.block];
     const int K = (MODE == 1) ? p.H : p.I;
 
-    // ---- copy plan: copy n of a stage lands at region (n >> 1), byte (n & 1) * 8 KB + wave * 1 KB + lane * 16.
-    // Byte o of a region holds piece q ^ (u & 3) of 4-row group u = o / 256, q = (row & 3) * 4 + piece.
+    // ---- copy plan: copy n of a stage lands at region n / 4, byte (n % 4) * 8 KB + wave * 1 KB + lane * 16.
+    // Byte o of a region holds piece q ^ (u & 7) of 2-row group u = o / 256, q = (row & 1) * 8 + piece.
     const uint16_t* src[kDmaPerStage];
     const uint16_t* wbase = (MODE == 1) ? p.w13 + static_cast<int64_t>(expert) * 2 * p.I * p.H
                                         : p.w2 + static_cast<int64_t>(expert) * p.H * p.I;
 #pragma unroll
     for (int n = 0; n < kDmaPerStage; ++n) {
-        const int o = (n & 1) * 8192 + wave * 1024 + lane * 16;
+        const int o = (n % kDmaHalf) * 8192 + wave * 1024 + lane * 16;
         const int u = o >> 8;
-        const int q = ((o >> 4) & 15) ^ (u & 3);
-        const int r = u * 4 + (q >> 2);
-        const int piece = q & 3;
-        if ((n >> 1) == 0) {
+        const int q = ((o >> 4) & 15) ^ (u & 7);
+        const int r = u * 2 + (q >> 3);
+        const int piece = q & 7;
+        if (n < kDmaHalf) {
             if (MODE == 1) {
                 const int slot = p.sorted_ids[m0 + r];
                 const int tok = (slot >= 0) ? slot / p.top_k : 0;
@@ -117,7 +122,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
         const int k0 = stage_k * kTK;
 #pragma unroll
         for (int n = 0; n < kDmaPerStage; ++n)
-            dma16(src[n] + k0, dma_base + buf * kStageBytes + (n >> 1) * kRegionBytes + (n & 1) * 8192);
+            dma16(src[n] + k0, dma_base + buf * kStageBytes + (n / kDmaHalf) * kRegionBytes + (n % kDmaHalf) * 8192);
     };
 
     f32x16_t acc[4][2];
@@ -131,41 +136,56 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
     // ---- operand reads: lane (r32, kh) takes row r32 of a 32-row fragment, piece ks*2 + kh ----
     const int r32 = lane & 31;
     const int kh = lane >> 5;
-    const int sw = (r32 >> 2) & 3;  // (row / 4) & 3 is the same for every fragment of this lane
-    int a_off[2], b_off[2];
+    const int sw = (r32 >> 1) & 7;  // (row / 2) & 7 is the same for every fragment of this lane
+    int a_off[4], b_off[4];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < 4; ++ks) {
         const int piece = (ks * 2 + kh) ^ sw;
         const int ra = wm * 128 + r32, rb = wn * 64 + r32;
-        a_off[ks] = (ra >> 2) * 256 + ((ra & 3) * 4 + piece) * 16;
-        b_off[ks] = kRegionBytes + (rb >> 2) * 256 + ((rb & 3) * 4 + piece) * 16;
+        a_off[ks] = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
+        b_off[ks] = kRegionBytes + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
     }
+    bf16x8_t fa[2][4], fb[2][2];
+    auto read_frags = [&](const uint8_t* s, int ks, int set) {
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) fa[set][mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off[ks] + mi * 4096);
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off[ks] + ni * 4096);
+    };
+    auto multiply = [&](int set) {
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
+        // scheduling hint: one LDS read after each of the first six MFMAs, then the last two MFMAs
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    };
 
     const int nk = K / kTK;
-#pragma unroll
-    for (int st = 0; st < kStages - 1; ++st)
-        if (st < nk) issue(st, st);
+    issue(0, 0);
+    wait_dma<0>();
+    block_barrier();
+    if (1 < nk) issue(1, 1);
+    read_frags(smem, 0, 0);
     for (int kt = 0; kt < nk; ++kt) {
-        // stage kt has landed once at most the copies of the (up to two) younger stages are in flight
-        if (kt + 2 < nk) wait_dma<2 * kDmaPerStage>();
-        else if (kt + 1 < nk) wait_dma<kDmaPerStage>();
-        else wait_dma<0>();
-        block_barrier();  // everyone's part of stage kt is in LDS; everyone is done reading stage kt-1
-        if (kt + kStages - 1 < nk) issue(kt + kStages - 1, (kt + kStages - 1) % kStages);
-        const uint8_t* s = smem + (kt % kStages) * kStageBytes;
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            bf16x8_t af[4], bfr[2];
-#pragma unroll
-            for (int mi = 0; mi < 4; ++mi) af[mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off[ks] + mi * 2048);
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni) bfr[ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off[ks] + ni * 2048);
-#pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], bfr[ni], acc[mi][ni], 0, 0, 0);
+        const uint8_t* s = smem + (kt & 1) * kStageBytes;
+        read_frags(s, 1, 1); multiply(0);
+        read_frags(s, 2, 0); multiply(1);
+        read_frags(s, 3, 1); multiply(0);
+        if (kt + 1 < nk) {
+            wait_dma<0>();                                   // this wave's part of stage kt+1 is in LDS
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of stage kt are in registers
+            block_barrier();                                 // ... and so are everyone else's
+            if (kt + 2 < nk) issue(kt + 2, kt & 1);          // stage kt's buffer is free again
+            read_frags(smem + ((kt + 1) & 1) * kStageBytes, 0, 0);
         }
+        multiply(1);
     }
 
     // ---- epilogue: element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
