@@ -39,6 +39,9 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=64, help="batch size T of the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run three device copies of 1 GiB (a plain copy kernel of known size that the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by)")
     return ap.parse_args()
 
 
@@ -154,6 +157,26 @@ def cpu_baseline(torch, T, w13, w2):
                       f"T={T} 8x7B batch, weights pre-cast to fp32, {sec * 1e3:.1f} ms per call"}
 
 
+def measured_traffic(T):
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration), or None."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(f"T{T}", {}).get("dominant_kernel_hbm_bytes")
+    except (OSError, ValueError):
+        return None
+
+
+def calibrate_copy(torch, dev):
+    src = torch.ones(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB read + 1 GiB written per copy
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -168,15 +191,25 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        calibrate_copy(torch, dev)
     w13, w2 = make_weights(torch, dev)
 
     T = args.tokens
     head = measure(torch, T, w13, w2, args.steps, args.warmup)
     g1_ms = head["stage_ms"]["gemm1"]
-    g1_bytes = head["n_active"] * 2 * I * H * 2 + T * H * 2   # w13 of the active experts + x
-    roofline = {"kernel": "w13 GEMM + SiLU*mul", "bound": "hbm", "achieved": g1_bytes / g1_ms / 1e6,
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": None,
-                "bytes_per_launch": g1_bytes, "avg_launch_ms": g1_ms}
+    if T <= 1024:
+        # decode: the w13 GEMM streams 2/3 of the weight bytes; HBM-bound
+        g1_bytes = head["n_active"] * 2 * I * H * 2 + T * H * 2   # w13 of the active experts + x
+        roofline = {"kernel": "w13 GEMM + SiLU*mul", "bound": "hbm", "achieved": g1_bytes / g1_ms / 1e6,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": measured_traffic(T),
+                    "per_launch": g1_bytes, "avg_launch_ms": g1_ms}
+    else:
+        # prefill: 4*H*I flops per routed slot in the w13 GEMM; MFMA-bound
+        g1_flops = T * TOPK * 4 * H * I
+        roofline = {"kernel": "w13 GEMM + SiLU*mul", "bound": "mfma", "achieved": g1_flops / g1_ms / 1e9,
+                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "traffic": measured_traffic(T),
+                    "per_launch": g1_flops, "avg_launch_ms": g1_ms}
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
 
     table = []
