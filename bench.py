@@ -39,6 +39,8 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=64, help="batch size T of the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
+    ap.add_argument("--accurate", action="store_true",
+                    help="run the layer with EM_FLAG_ACCURATE (bf16 hi+lo activations through the w2 GEMM)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three device copies of 1 GiB (a plain copy kernel of known size that the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by)")
@@ -71,6 +73,8 @@ def make_batch(torch, dev, T, seed=0, logits="normal"):
 class LayerRunner:
     """Calls em_moe_forward through the C ABI with pre-allocated buffers."""
 
+    base_flags = 0
+
     def __init__(self, torch, T, w13, w2, x, lg):
         import ctypes
         from electrock_infer_amd import _lib
@@ -85,7 +89,7 @@ class LayerRunner:
         code = self.lib.em_moe_forward(
             self.x.data_ptr(), self.lg.data_ptr(), self._lib.DTYPE_BF16, self.w13.data_ptr(), self.w2.data_ptr(),
             self.out.data_ptr(), self.T, H, I, E, TOPK, 1, self.ws.buffer.data_ptr(),
-            self.ctypes.c_size_t(self.ws.buffer.numel()), flags,
+            self.ctypes.c_size_t(self.ws.buffer.numel()), flags | self.base_flags,
             self.torch.cuda.current_stream().cuda_stream)
         self._lib.check(code, "em_moe_forward")
 
@@ -191,6 +195,8 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.accurate:
+        LayerRunner.base_flags = _lib.FLAG_ACCURATE
     if args.calibrate_copy:
         calibrate_copy(torch, dev)
     w13, w2 = make_weights(torch, dev)
@@ -231,7 +237,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"Mixtral-8x7B MoE layer decode T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
                                f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
-                   "tokens": T, "n_active_experts": head["n_active"]},
+                   "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate)},
         "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(torch, T, w13, w2),

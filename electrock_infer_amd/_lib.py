@@ -14,6 +14,7 @@ DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 ITYPE_I32, ITYPE_I64 = 0, 1
 
 FLAG_OUT_F32 = 1 << 0
+FLAG_ACCURATE = 1 << 1
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10
@@ -33,7 +34,7 @@ class MoeLayout(ctypes.Structure):
     """Mirror of struct em_moe_layout."""
     _fields_ = [(n, ctypes.c_int64) for n in (
         "block_size", "topk_weights_off", "topk_ids_off", "sorted_ids_off", "sorted_len",
-        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "act_off", "y_off", "ksplit",
+        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "act_off", "act_lo_off", "y_off", "ksplit",
         "total_bytes")]
 
 

@@ -124,6 +124,7 @@ int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_la
     L->post_pad_off = take(4);
     L->seg_begin_off = take((E + 1) * 4);
     L->act_off = take(sorted_len * static_cast<int64_t>(I) * 2);
+    L->act_lo_off = take(sorted_len * static_cast<int64_t>(I) * 2);
     L->ksplit = choose_ksplit(T, I);
     L->y_off = take(L->ksplit * slots * static_cast<int64_t>(H) * 4);
     L->total_bytes = off;
@@ -158,6 +159,9 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
     p.w13 = static_cast<const uint16_t*>(w13);
     p.w2 = static_cast<const uint16_t*>(w2);
     p.act = reinterpret_cast<uint16_t*>(ws + L.act_off);
+    const bool accurate = (flags & EM_FLAG_ACCURATE) != 0;
+    p.act_lo = accurate ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
+    p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
     int32_t* eids = reinterpret_cast<int32_t*>(ws + L.expert_ids_off);
@@ -195,8 +199,18 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
-        rc = use_stream ? launch_gemm_stream(p, seg_begin, 2, s)
-             : use_tile ? launch_gemm_tile(p, 2, s) : launch_gemm_generic(p, 2, s);
+        if (use_stream) {
+            rc = launch_gemm_stream(p, seg_begin, 2, s);  // multiplies act and act_lo in one pass
+        } else {
+            rc = use_tile ? launch_gemm_tile(p, 2, s) : launch_gemm_generic(p, 2, s);
+            if (rc == 0 && accurate) {  // second pass: y += act_lo . w2
+                MoeProblem lo = p;
+                lo.act = p.act_lo;
+                lo.act_lo = nullptr;
+                lo.y_accumulate = 1;
+                rc = use_tile ? launch_gemm_tile(lo, 2, s) : launch_gemm_generic(lo, 2, s);
+            }
+        }
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_COMBINE)) {

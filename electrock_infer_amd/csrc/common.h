@@ -84,6 +84,8 @@ struct MoeProblem {
     const uint16_t* w13;      // [E, 2I, H] bf16
     const uint16_t* w2;       // [E, H, I] bf16
     uint16_t* act;            // [sorted_len, I] bf16, rows in sorted (padded) order
+    uint16_t* act_lo;         // same shape: bf16(value - act) in accurate mode, else null
+    int y_accumulate;         // w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
     const int32_t* sorted_ids;
     const int32_t* expert_ids;
@@ -95,6 +97,13 @@ struct MoeProblem {
     int64_t sorted_len;       // worst-case padded length
     int ksplit;
 };
+// SiLU*mul result -> act (and the rounding residual -> act_lo in accurate mode)
+__device__ __forceinline__ void store_act(const MoeProblem& p, int64_t idx, float v) {
+    const uint16_t hi = f32_to_bf16_bits(v);
+    p.act[idx] = hi;
+    if (p.act_lo != nullptr) p.act_lo[idx] = f32_to_bf16_bits(v - bf16_bits_to_f32(hi));
+}
+
 int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s);  // mode 1: w13+SiLU*mul, 2: w2
 bool stream_supported(const MoeProblem& p);
 int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s);

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(MoeProblem p) {
                     const float g = acc[f][0][v];
                     const float u = acc[f][1][v];
                     const float s = g / (1.0f + __expf(-g));
-                    p.act[(m0 + f * 16 + kq * 4 + v) * static_cast<int64_t>(p.I) + j] = f32_to_bf16_bits(s * u);
+                    store_act(p, (m0 + f * 16 + kq * 4 + v) * static_cast<int64_t>(p.I) + j, s * u);
                 }
         }
     } else {
@@ -177,7 +177,10 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(MoeProblem p) {
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const int n = n0 + wave * 32 + h * 16 + r16;
-                    if (n < Nw) ybase[static_cast<int64_t>(slot) * p.H + n] = acc[f][h][v];
+                    if (n < Nw) {
+                        float* dst = ybase + static_cast<int64_t>(slot) * p.H + n;
+                        *dst = p.y_accumulate ? *dst + acc[f][h][v] : acc[f][h][v];
+                    }
                 }
             }
     }

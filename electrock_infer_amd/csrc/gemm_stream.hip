@@ -40,7 +40,9 @@ __device__ __forceinline__ u32x4_t ld16_stream(const uint16_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
 }
 
-template <int MODE>
+// LO: the token rows exist as a bf16 pair act + act_lo (accurate mode, MODE 2 only); both halves are
+// multiplied with the same weight fragments, which costs no extra weight traffic.
+template <int MODE, bool LO>
 __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem p,
                                                                      const int32_t* __restrict__ seg_begin,
                                                                      int tiles_per_expert, int kslice) {
@@ -91,6 +93,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 
         // token rows of this lane (operand layout: row r16 of each fragment)
         const uint16_t* arow[kMaxF];
+        int64_t lo_delta = 0;  // element offset from an act row to the same row of act_lo
+        if (LO) lo_delta = p.act_lo - p.act;
 #pragma unroll
         for (int f = 0; f < kMaxF; ++f) {
             arow[f] = nullptr;
@@ -111,18 +115,21 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 #pragma unroll
             for (int g = 0; g < 4; ++g) acc[f][g] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-        u32x4_t b0[8], b1[8], a0[kMaxF][2], a1[kMaxF][2];
-        auto issue = [&](int s, u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][2]) {
+        constexpr int kAW = LO ? 4 : 2;  // per fragment: two 32-wide K halves (x2 with the low parts)
+        u32x4_t b0[8], b1[8], a0[kMaxF][kAW], a1[kMaxF][kAW];
+        auto issue = [&](int s, u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][kAW]) {
             const int koff = s * kStep;
 #pragma unroll
             for (int i = 0; i < 8; ++i) b[i] = ld16_stream(brow[i] + koff);
 #pragma unroll
             for (int f = 0; f < kMaxF; ++f)
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+                for (int ks = 0; ks < 2; ++ks) {
                     a[f][ks] = (arow[f] != nullptr) ? ld16(arow[f] + koff + ks * 32) : u32x4_t{0, 0, 0, 0};
+                    if (LO) a[f][2 + ks] = (arow[f] != nullptr) ? ld16(arow[f] + lo_delta + koff + ks * 32) : u32x4_t{0, 0, 0, 0};
+                }
         };
-        auto consume = [&](u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][2]) {
+        auto consume = [&](u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][kAW]) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 *reinterpret_cast<u32x4_t*>(my + (i * 8 + lrow) * kPitch + lchunk * 16) = b[i];
@@ -140,6 +147,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
                             acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[g], acc[f][g], 0, 0, 0);
+                        if (LO) {
+                            __builtin_memcpy(&af, &a[f][2 + ks], 16);
+#pragma unroll
+                            for (int g = 0; g < 4; ++g)
+                                acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[g], acc[f][g], 0, 0, 0);
+                        }
                     }
                 }
             }
@@ -180,7 +193,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
                     for (int v = 0; v < 4; ++v) {
                         const float s = g[v] / (1.0f + __expf(-g[v]));
                         const int64_t row = seg + (f0 + f) * 16 + kq * 4 + v;
-                        p.act[row * p.I + j] = f32_to_bf16_bits(s * u[v]);
+                        store_act(p, row * p.I + j, s * u[v]);
                     }
                 }
             }
@@ -213,12 +226,15 @@ int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, 
     const dim3 blk(kWaves * 64);
     if (mode == 1) {
         const int tiles = p.I / 32;
-        hipLaunchKernelGGL(gemm_stream_kernel<1>, dim3(static_cast<unsigned>(p.E * tiles), 1), blk, 0, s, p, seg_begin,
-                           tiles, p.H);
+        hipLaunchKernelGGL((gemm_stream_kernel<1, false>), dim3(static_cast<unsigned>(p.E * tiles), 1), blk, 0, s, p,
+                           seg_begin, tiles, p.H);
     } else {
         const int tiles = p.H / kRows;
-        hipLaunchKernelGGL(gemm_stream_kernel<2>, dim3(static_cast<unsigned>(p.E * tiles), static_cast<unsigned>(p.ksplit)),
-                           blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
+        const dim3 grid(static_cast<unsigned>(p.E * tiles), static_cast<unsigned>(p.ksplit));
+        if (p.act_lo != nullptr)
+            hipLaunchKernelGGL((gemm_stream_kernel<2, true>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
+        else
+            hipLaunchKernelGGL((gemm_stream_kernel<2, false>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
     }
     return launch_status();
 }

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
                 const float g = acc[mi][0][v];
                 const float u = acc[mi][1][v];
                 const float sg = g / (1.0f + __expf(-g));
-                p.act[(m0 + row) * static_cast<int64_t>(p.I) + j] = f32_to_bf16_bits(sg * u);
+                store_act(p, (m0 + row) * static_cast<int64_t>(p.I) + j, sg * u);
             }
     } else {
 #pragma unroll
@@ -210,8 +210,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
                 const int slot = p.sorted_ids[m0 + row];
                 if (slot < 0) continue;
                 float* yrow = p.y + static_cast<int64_t>(slot) * p.H + nt * kTN + wn * 64 + r32;
-                yrow[0] = acc[mi][0][v];
-                yrow[32] = acc[mi][1][v];
+                yrow[0] = p.y_accumulate ? yrow[0] + acc[mi][0][v] : acc[mi][0][v];
+                yrow[32] = p.y_accumulate ? yrow[32] + acc[mi][1][v] : acc[mi][1][v];
             }
     }
 }

@@ -97,7 +97,7 @@ def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int) -> MoeWork
 def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
                   gating_output: torch.Tensor, topk: int, renormalize: bool = True,
                   inplace: bool = False, activation: str = "silu",
-                  out_dtype: Optional[torch.dtype] = None, flags: int = 0,
+                  out_dtype: Optional[torch.dtype] = None, accurate: bool = False, flags: int = 0,
                   workspace: Optional[MoeWorkspace] = None) -> torch.Tensor:
     """The MoE layer body (fused_moe.py:170-293): route, sort, w13 GEMM with
     SiLU*mul, w2 GEMM, weighted top-k combine.
@@ -106,7 +106,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     gating_output [T, E].  With ``inplace`` the result overwrites
     ``hidden_states`` and that tensor is returned, as in the reference.
     ``out_dtype=torch.float32`` returns the un-rounded fp32 result instead
-    (not available together with ``inplace``).
+    (not available together with ``inplace``).  ``accurate=True`` keeps the
+    SiLU*mul activations as a bf16 hi+lo pair through the w2 GEMM.
     """
     if activation != "silu":
         raise NotImplementedError(f"Activation {activation} not supported.")
@@ -121,6 +122,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     if not (hidden_states.dtype == w1.dtype == w2.dtype == torch.bfloat16):
         raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, w1 and w2 must be bfloat16")
     want_f32 = out_dtype == torch.float32
+    if accurate:
+        flags |= _lib.FLAG_ACCURATE
     if want_f32 and inplace:
         raise RuntimeError("a float32 result cannot be written in place over bfloat16 hidden_states")
     if want_f32:

@@ -44,6 +44,7 @@ extern "C" {
 
 /* em_moe_forward flags */
 #define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16      */
+#define EM_FLAG_ACCURATE       (1u << 1)  /* SiLU*mul activations kept as a bf16 hi+lo pair  */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
 #define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
 #define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
@@ -139,6 +140,11 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  *   w2            [E, H, I]   bf16 (mixtral_moe.py:75-79)
  *   out           [T, H]      bf16 (float32 with EM_FLAG_OUT_F32); may alias x
  *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k), 256-byte aligned
+ * EM_FLAG_ACCURATE keeps the SiLU*mul activations as a bf16 pair (value, rounding
+ * residual) and multiplies both with w2, which removes the one rounding the bf16 MFMA
+ * of the w2 GEMM otherwise needs; together with EM_FLAG_OUT_F32 the result is within
+ * fp32 accumulation error of the fp32 definition.  Free for T <= 64 (the layer is
+ * HBM-bound there), one extra w2 pass otherwise.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.
@@ -162,6 +168,7 @@ typedef struct em_moe_layout {
     int64_t post_pad_off;                          /* [1] i32                  */
     int64_t seg_begin_off;                         /* [E+1] i32 padded segment starts */
     int64_t act_off;                               /* [sorted_len, I] bf16     */
+    int64_t act_lo_off;                            /* [sorted_len, I] bf16, accurate mode */
     int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 */
     int64_t total_bytes;
 } em_moe_layout;

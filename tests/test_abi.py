@@ -67,9 +67,9 @@ def test_workspace_layout_is_consistent():
         assert L.sorted_len % L.block_size == 0 and L.sorted_len >= T * 2 + 8 * (L.block_size - 1)
         assert L.expert_ids_len * L.block_size == L.sorted_len
         offs = [L.topk_weights_off, L.topk_ids_off, L.sorted_ids_off, L.expert_ids_off, L.post_pad_off,
-                L.act_off, L.y_off, L.total_bytes]
+                L.act_off, L.act_lo_off, L.y_off, L.total_bytes]
         assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
-        assert L.y_off - L.act_off >= L.sorted_len * I * 2
+        assert L.act_lo_off - L.act_off >= L.sorted_len * I * 2 and L.y_off - L.act_lo_off >= L.sorted_len * I * 2
         assert L.total_bytes - L.y_off >= L.ksplit * T * 2 * H * 4
     assert lib.em_moe_workspace_bytes(4, 4097, 512, 8, 2) == 0
 
