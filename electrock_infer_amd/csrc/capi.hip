@@ -16,17 +16,23 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 // couple of MFMA fragments per expert); above it the tiled kernels take over.
 constexpr int64_t kStreamMaxT = 64;
 
-// Counterpart of _get_moe_config (fused_moe.py:327-339): rows per sorted block.
-// An expert receives at most T rows, so up to 16 tokens one 16-row MFMA
-// fragment per expert always suffices.
-// From this many tokens on (>= 256 rows per expert on average for 8 experts, top-2)
-// the 256 x 256 tiled kernel runs and the sort pads experts to 256 rows.
-constexpr int64_t kTileMinT = 1024;
-inline int choose_block(int64_t T) { return T <= kStreamMaxT ? 16 : (T < kTileMinT ? 64 : 256); }
+// Rows per sorted block, the counterpart of _get_moe_config (fused_moe.py:327-339):
+// 16 (one MFMA fragment) for the streaming kernel, 32 for the tiled kernel, which cuts
+// experts into tiles of up to 256 rows itself, 64 for the generic kernel.
+inline int choose_block(int64_t T, int H, int I) {
+    if (T <= kStreamMaxT) return 16;
+    return tile_shape_ok(H, I) ? tile_row_block() : 64;
+}
 // Split of the w2 reduction (K = I) across workgroups for small batches, where
-// (row blocks) x (H / 128 column tiles) alone would leave most CUs idle.
-inline int choose_ksplit(int64_t T, int I) {
-    if (T > kStreamMaxT) return T <= 512 ? 4 : 1;
+// (row tiles) x (column tiles) alone would leave most CUs idle.
+inline int choose_ksplit(int64_t T, int H, int I) {
+    if (T > kStreamMaxT) {
+        const int want = T <= 512 ? 4 : 1;
+        if (!tile_shape_ok(H, I)) return want;
+        for (int ks = want; ks >= 1; --ks)  // the tiled kernel needs I / ksplit to be a multiple of 64
+            if (I % (ks * 64) == 0) return ks;
+        return 1;
+    }
     // Streaming kernel: (active experts) x (H / 64) row tiles should give every CU
     // work.  From ~17 tokens on all eight experts are almost surely active and one
     // K slice per tile measures fastest; below that the reduction is split four ways.
@@ -105,7 +111,7 @@ int em_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dt
 int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_layout* L) {
     if (!L) return EM_ERR_NULL_POINTER;
     if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
-    const int64_t block = choose_block(T);
+    const int64_t block = choose_block(T, H, I);
     const int64_t slots = T * top_k;
     const int64_t sorted_len = round_up(slots + static_cast<int64_t>(E) * (block - 1), block);
     int64_t off = 0;
@@ -125,7 +131,7 @@ int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_la
     L->seg_begin_off = take((E + 1) * 4);
     L->act_off = take(sorted_len * static_cast<int64_t>(I) * 2);
     L->act_lo_off = take(sorted_len * static_cast<int64_t>(I) * 2);
-    L->ksplit = choose_ksplit(T, I);
+    L->ksplit = choose_ksplit(T, H, I);
     L->y_off = take(L->ksplit * slots * static_cast<int64_t>(H) * 4);
     L->total_bytes = off;
     return 0;
@@ -192,23 +198,23 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
         if (rc != 0) return rc;
     }
     const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
-    const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T >= kTileMinT && tile_supported(p);
+    const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T > kStreamMaxT && tile_supported(p);
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
         rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s)
-             : use_tile ? launch_gemm_tile(p, 1, s) : launch_gemm_generic(p, 1, s);
+             : use_tile ? launch_gemm_tile(p, seg_begin, 1, s) : launch_gemm_generic(p, 1, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
         if (use_stream) {
             rc = launch_gemm_stream(p, seg_begin, 2, s);  // multiplies act and act_lo in one pass
         } else {
-            rc = use_tile ? launch_gemm_tile(p, 2, s) : launch_gemm_generic(p, 2, s);
+            rc = use_tile ? launch_gemm_tile(p, seg_begin, 2, s) : launch_gemm_generic(p, 2, s);
             if (rc == 0 && accurate) {  // second pass: y += act_lo . w2
                 MoeProblem lo = p;
                 lo.act = p.act_lo;
                 lo.act_lo = nullptr;
                 lo.y_accumulate = 1;
-                rc = use_tile ? launch_gemm_tile(lo, 2, s) : launch_gemm_generic(lo, 2, s);
+                rc = use_tile ? launch_gemm_tile(lo, seg_begin, 2, s) : launch_gemm_generic(lo, 2, s);
             }
         }
         if (rc != 0) return rc;

@@ -107,8 +107,10 @@ __device__ __forceinline__ void store_act(const MoeProblem& p, int64_t idx, floa
 int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s);  // mode 1: w13+SiLU*mul, 2: w2
 bool stream_supported(const MoeProblem& p);
 int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s);
+bool tile_shape_ok(int H, int I);
+int tile_row_block();
 bool tile_supported(const MoeProblem& p);
-int launch_gemm_tile(const MoeProblem& p, int mode, hipStream_t s);
+int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s);
 int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s);
 
 }  // namespace em

@@ -1,13 +1,24 @@
-// Tiled grouped expert GEMM for prefill batches (hundreds of rows per expert),
-// where the layer is bound by the bf16 MFMA rate.
+// Tiled grouped expert GEMM for batches beyond decode size (tens to thousands of rows
+// per expert), where the layer moves from HBM-bound to bound by the bf16 MFMA rate.
 //
-//   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile 256 sorted rows x 256
+//   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile of up to 256 sorted rows x 256
 //              weight rows; K in steps of 64 through two 64 KB LDS stages
+//   tiles      the sort pads experts to 32 rows only; every expert is cut into 256-row
+//              tiles and its last tile is as high as the rows that are left (a multiple
+//              of 32).  A wave multiplies only the 32-row fragments that exist, so a
+//              short tile costs its share of MFMA time, and its missing A rows are not
+//              fetched.  The tile list is rebuilt by every workgroup from the per-expert
+//              segment starts (at most 64 scalar loads).
 //   loads      global -> LDS directly (global_load_lds_dwordx4), no registers in
 //              between; eight lanes fetch one full 128-byte line of a row (measured
 //              L2 -> CU feed: ~23 TB/s with 128 B per row against ~16 TB/s with 64 B);
 //              the copy of stage k+1 runs while stage k is multiplied; completion is
 //              tracked by hand with s_waitcnt vmcnt + one s_barrier per stage
+//   prefetch   a stage only completes when its slowest line has arrived, and the first
+//              workgroup of an XCD to ask for a line pays HBM latency; so every
+//              workgroup also touches (one dword per line, into a dummy LDS area) its
+//              share of the lines that the workgroups sharing its A and B tiles will
+//              need six stages later, which turns those misses into L2 hits
 //   LDS        rows are 128 B; the 16-byte pieces of every 2-row group are XOR-
 //              swizzled so that the 16 lanes of a b128 operand read hit 16 bank groups
 //   wave       128 x 64 sub-tile = 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (the
@@ -16,16 +27,14 @@
 //              MFMAs of the previous 16-wide K step, also across the stage barrier
 //   MODE 1     the wave's two N fragments are 32 gate rows j and the matching 32
 //              up rows I + j, so SiLU(g) * u is lane-local in the epilogue
-//   MODE 2     256 rows of w2[e]; fp32 partial rows are scattered to y[slot]
-//   rows       A rows are gathered through sorted_token_ids (MODE 1) or read in
-//              sorted order from act (MODE 2); the sort pads every expert to 256.
-//              Pad rows read token 0: their products only reach pad rows of act,
-//              which no output row depends on.
+//   MODE 2     256 rows of w2[e], optionally one of `ksplit` K slices; fp32 partial rows
+//              are scattered to y[z, slot]
 //   order      workgroup ids are dealt to the 8 XCDs round-robin by the hardware;
 //              they are re-mapped so that each XCD walks one contiguous range of
-//              tiles, ordered 4 row blocks x all column tiles, which lets the 32
+//              tiles, ordered 4 row tiles x all column tiles, which lets the 32
 //              CUs of an XCD share A and B tiles through their own L2.
 #include "common.h"
+#include <type_traits>
 
 namespace em {
 namespace {
@@ -36,6 +45,9 @@ constexpr int kStages = 2;
 constexpr int kRegionBytes = kTM * kTK * 2;          // 32 KB: A rows, then 32 KB of B rows
 constexpr int kStageBytes = 2 * kRegionBytes;        // 64 KB
 constexpr int kLdsBytes = kStages * kStageBytes;     // 128 KB
+constexpr int kTouchBytes = 8 * 256;                 // dummy landing area of the L2 touches
+constexpr int kTouchAhead = 6;                       // stages between a touch and its use
+constexpr int kRowBlock = 32;                        // sort padding this kernel needs
 constexpr int kGroupM = 4;
 constexpr int kXcds = 8;
 constexpr int kDmaPerStage = kStageBytes / (kThreads * 16);  // 8 per thread
@@ -57,15 +69,23 @@ template <int N>
 __device__ __forceinline__ void wait_dma() {  // at most N of this wave's copies still in flight
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
+// Same for one dword per lane (256 B of LDS per wave): used only to pull lines into L2.
+__device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                 :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
 __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 template <int MODE>
-__global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, int ntiles_n) {
+__global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
+                                                               int ntiles_n, int kslice) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-    // ---- which tile: XCD-aware re-mapping over the ACTUAL number of row blocks ----
-    const int mblocks = p.post_pad[0] / kTM;
-    const int total = mblocks * ntiles_n;
+    // ---- tile list: expert e owns ceil(rows_e / 256) row tiles ----
+    int mtiles = 0;
+    for (int e = 0; e < p.E; ++e) mtiles += (seg_begin[e + 1] - seg_begin[e] + kTM - 1) / kTM;
+    // ---- which tile: XCD-aware re-mapping over the ACTUAL number of row tiles ----
+    const int total = mtiles * ntiles_n;
     const int per_xcd = (total + kXcds - 1) / kXcds;
     const int xcd = blockIdx.x % kXcds;
     const int local = blockIdx.x / kXcds;
@@ -74,22 +94,33 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
     const int group_sz = kGroupM * ntiles_n;
     const int group = logical / group_sz;
     const int in_group = logical - group * group_sz;
-    const int rows_in_group = (mblocks - group * kGroupM < kGroupM) ? mblocks - group * kGroupM : kGroupM;
-    const int mb = group * kGroupM + in_group % rows_in_group;
+    const int rows_in_group = (mtiles - group * kGroupM < kGroupM) ? mtiles - group * kGroupM : kGroupM;
+    const int m_in_group = in_group % rows_in_group;
     const int nt = in_group / rows_in_group;
+    int mt = group * kGroupM + m_in_group;  // global row-tile index -> (expert, tile inside the expert)
+    int expert = 0;
+    for (; expert < p.E - 1; ++expert) {
+        const int t = (seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM;
+        if (mt < t) break;
+        mt -= t;
+    }
+    const int64_t m0 = seg_begin[expert] + static_cast<int64_t>(mt) * kTM;
+    const int rows_left = seg_begin[expert + 1] - static_cast<int>(m0);
+    const int valid = rows_left < kTM ? rows_left : kTM;  // multiple of 32, >= 32
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave >> 2;  // 0..1
     const int wn = wave & 3;   // 0..3
-    const int64_t m0 = static_cast<int64_t>(mb) * kTM;
-    const int expert = p.expert_ids[m0 / p.block];
     const int K = (MODE == 1) ? p.H : p.I;
+    const int k_begin = blockIdx.y * kslice;
 
     // ---- copy plan: copy n of a stage lands at region n / 4, byte (n % 4) * 8 KB + wave * 1 KB + lane * 16.
     // Byte o of a region holds piece q ^ (u & 7) of 2-row group u = o / 256, q = (row & 1) * 8 + piece.
+    // One copy covers 8 whole rows; copies of A rows beyond `valid` are skipped.
     const uint16_t* src[kDmaPerStage];
+    bool live[kDmaPerStage];
     const uint16_t* wbase = (MODE == 1) ? p.w13 + static_cast<int64_t>(expert) * 2 * p.I * p.H
                                         : p.w2 + static_cast<int64_t>(expert) * p.H * p.I;
 #pragma unroll
@@ -100,20 +131,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
         const int r = u * 2 + (q >> 3);
         const int piece = q & 7;
         if (n < kDmaHalf) {
+            live[n] = ((n % kDmaHalf) * 64 + wave * 8) < valid;  // wave-uniform
+            const int rr = (r < valid) ? r : 0;
             if (MODE == 1) {
-                const int slot = p.sorted_ids[m0 + r];
-                const int tok = (slot >= 0) ? slot / p.top_k : 0;
-                src[n] = p.x + static_cast<int64_t>(tok) * p.H + piece * 8;
+                const int slot = p.sorted_ids[m0 + rr];
+                const int tok = (slot >= 0) ? slot / p.top_k : 0;  // pad rows multiply token 0; never stored
+                src[n] = p.x + static_cast<int64_t>(tok) * p.H + k_begin + piece * 8;
             } else {
-                src[n] = p.act + (m0 + r) * static_cast<int64_t>(p.I) + piece * 8;
+                src[n] = p.act + (m0 + rr) * static_cast<int64_t>(p.I) + k_begin + piece * 8;
             }
         } else {
+            live[n] = true;
             int64_t grow;
             if (MODE == 1)  // LDS row r of the B tile: wave column r/64, gate (0) or up (1) half, j offset r%32
                 grow = static_cast<int64_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31);
             else
                 grow = static_cast<int64_t>(nt) * kTN + r;
-            src[n] = wbase + grow * K + piece * 8;
+            src[n] = wbase + grow * K + k_begin + piece * 8;
         }
     }
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
@@ -122,7 +156,40 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
         const int k0 = stage_k * kTK;
 #pragma unroll
         for (int n = 0; n < kDmaPerStage; ++n)
-            dma16(src[n] + k0, dma_base + buf * kStageBytes + (n / kDmaHalf) * kRegionBytes + (n % kDmaHalf) * 8192);
+            if (live[n])
+                dma16(src[n] + k0, dma_base + buf * kStageBytes + (n / kDmaHalf) * kRegionBytes + (n % kDmaHalf) * 8192);
+    };
+
+    // ---- L2 touch plan: line id = wave * 64 + lane, 0..255 = A rows, 256..511 = B rows.  The up to 8 column
+    // tiles that run next to this one share its A tile and the 4 row tiles of its group share its B tile, so
+    // this workgroup touches every 8th A line and every 4th B line; other lanes repeat line 0 (coalesced away).
+    // Every wave issues exactly one touch per stage, which keeps the vmcnt bookkeeping uniform.
+    const uint16_t* touch_src;
+    {
+        const int tl = wave * 64 + lane;
+        const int trow = tl & 255;
+        if (tl < 256) {
+            const bool mine = (trow & 7) == (nt & 7) && trow < valid;
+            const int rr = mine ? trow : 0;
+            if (MODE == 1) {
+                const int slot = p.sorted_ids[m0 + rr];
+                touch_src = p.x + static_cast<int64_t>(slot >= 0 ? slot / p.top_k : 0) * p.H + k_begin;
+            } else {
+                touch_src = p.act + (m0 + rr) * static_cast<int64_t>(p.I) + k_begin;
+            }
+        } else {
+            const bool mine = (trow & 3) == m_in_group;
+            const int r = mine ? trow : 0;
+            const int64_t grow = (MODE == 1)
+                                     ? static_cast<int64_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31)
+                                     : static_cast<int64_t>(nt) * kTN + r;
+            touch_src = wbase + grow * K + k_begin;
+        }
+    }
+    const uint32_t touch_dst = __builtin_amdgcn_readfirstlane(lds0 + kLdsBytes + wave * 256);
+    const int nk = kslice / kTK;
+    auto touch = [&](int stage_k) {
+        dma4(touch_src + (stage_k < nk ? stage_k : nk - 1) * kTK, touch_dst);
     };
 
     f32x16_t acc[4][2];
@@ -145,54 +212,82 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
         a_off[ks] = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
         b_off[ks] = kRegionBytes + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
     }
-    bf16x8_t fa[2][4], fb[2][2];
-    auto read_frags = [&](const uint8_t* s, int ks, int set) {
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) fa[set][mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off[ks] + mi * 4096);
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off[ks] + ni * 4096);
-    };
-    auto multiply = [&](int set) {
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
-        // scheduling hint: one LDS read after each of the first six MFMAs, then the last two MFMAs
-#pragma unroll
-        for (int i = 0; i < 6; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-    };
+    // 32-row fragments of this wave that hold rows of the tile (wave-uniform)
+    int nmi = (valid - wm * 128 + 31) / 32;
+    nmi = nmi < 0 ? 0 : (nmi > 4 ? 4 : nmi);
+    nmi = __builtin_amdgcn_readfirstlane(nmi);
 
-    const int nk = K / kTK;
-    issue(0, 0);
-    wait_dma<0>();
-    block_barrier();
-    if (1 < nk) issue(1, 1);
-    read_frags(smem, 0, 0);
-    for (int kt = 0; kt < nk; ++kt) {
-        const uint8_t* s = smem + (kt & 1) * kStageBytes;
-        read_frags(s, 1, 1); multiply(0);
-        read_frags(s, 2, 0); multiply(1);
-        read_frags(s, 3, 1); multiply(0);
-        if (kt + 1 < nk) {
-            wait_dma<0>();                                   // this wave's part of stage kt+1 is in LDS
+    bf16x8_t fa[2][4], fb[2][2];
+    // FULL: all four fragments exist (the common case) -> fixed instruction mix with scheduling hints
+    auto main_loop = [&](auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        auto read_frags = [&](const uint8_t* s, int ks, int set) {
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+                if (FULL || mi < nmi) fa[set][mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off[ks] + mi * 4096);
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off[ks] + ni * 4096);
+        };
+        auto multiply = [&](int set) {
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+                if (FULL || mi < nmi) {
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
+                }
+            if (FULL) {  // scheduling hint: one LDS read after each of the first six MFMAs, then the last two
+#pragma unroll
+                for (int i = 0; i < 6; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+        };
+        const bool work = FULL || nmi > 0;  // waves without rows still copy, touch and meet the barriers
+        issue(0, 0);
+        touch(1);
+        wait_dma<1>();  // everything but the touch
+        block_barrier();
+        if (1 < nk) issue(1, 1);
+        touch(2);
+        if (work) read_frags(smem, 0, 0);
+        for (int kt = 0; kt + 1 < nk; ++kt) {
+            const uint8_t* s = smem + (kt & 1) * kStageBytes;
+            if (work) {
+                read_frags(s, 1, 1); multiply(0);
+                read_frags(s, 2, 0); multiply(1);
+                read_frags(s, 3, 1); multiply(0);
+            }
+            wait_dma<1>();                                      // this wave's part of stage kt+1 is in LDS
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of stage kt are in registers
-            block_barrier();                                 // ... and so are everyone else's
-            if (kt + 2 < nk) issue(kt + 2, kt & 1);          // stage kt's buffer is free again
-            read_frags(smem + ((kt + 1) & 1) * kStageBytes, 0, 0);
+            block_barrier();                                    // ... and so are everyone else's
+            if (kt + 2 < nk) issue(kt + 2, kt & 1);             // stage kt's buffer is free again
+            touch(kt + 2 + kTouchAhead);
+            if (work) {
+                read_frags(smem + ((kt + 1) & 1) * kStageBytes, 0, 0);
+                multiply(1);
+            }
         }
-        multiply(1);
-    }
+        if (work) {  // last stage: nothing left to copy
+            const uint8_t* s = smem + ((nk - 1) & 1) * kStageBytes;
+            read_frags(s, 1, 1); multiply(0);
+            read_frags(s, 2, 0); multiply(1);
+            read_frags(s, 3, 1); multiply(0);
+            multiply(1);
+        }
+        wait_dma<0>();  // the last touches must not outlive the workgroup's LDS
+    };
+    if (nmi == 4) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
 
     // ---- epilogue: element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
     if (MODE == 1) {
         const int j = nt * 128 + wn * 32 + r32;
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+        for (int mi = 0; mi < 4; ++mi) {
+            if (mi >= nmi) break;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
@@ -201,35 +296,44 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, in
                 const float sg = g / (1.0f + __expf(-g));
                 store_act(p, (m0 + row) * static_cast<int64_t>(p.I) + j, sg * u);
             }
+        }
     } else {
+        float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H;
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+        for (int mi = 0; mi < 4; ++mi) {
+            if (mi >= nmi) break;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
                 const int slot = p.sorted_ids[m0 + row];
                 if (slot < 0) continue;
-                float* yrow = p.y + static_cast<int64_t>(slot) * p.H + nt * kTN + wn * 64 + r32;
+                float* yrow = ybase + static_cast<int64_t>(slot) * p.H + nt * kTN + wn * 64 + r32;
                 yrow[0] = p.y_accumulate ? yrow[0] + acc[mi][0][v] : acc[mi][0][v];
                 yrow[32] = p.y_accumulate ? yrow[32] + acc[mi][1][v] : acc[mi][1][v];
             }
+        }
     }
 }
 
 }  // namespace
 
+bool tile_shape_ok(int H, int I) { return H % kTN == 0 && I % 128 == 0 && H % kTK == 0 && I % kTK == 0; }
+int tile_row_block() { return kRowBlock; }
+
 bool tile_supported(const MoeProblem& p) {
-    return p.block == kTM && p.ksplit == 1 && p.H % kTN == 0 && p.I % 128 == 0 && p.H % kTK == 0 &&
-           p.I % kTK == 0 && p.T > 0;
+    return p.block == kRowBlock && tile_shape_ok(p.H, p.I) && p.T > 0 && p.ksplit >= 1 &&
+           p.I % (p.ksplit * kTK) == 0;
 }
 
-int launch_gemm_tile(const MoeProblem& p, int mode, hipStream_t s) {
+int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s) {
     if (!tile_supported(p)) return EM_ERR_UNSUPPORTED;
     const int ntiles_n = (mode == 1) ? p.I / 128 : p.H / kTN;
-    const int64_t max_mblocks = p.sorted_len / kTM;
-    const int64_t total = max_mblocks * ntiles_n;
+    // upper bound of the sum over experts of ceil(padded rows_e / 256)
+    const int64_t max_mtiles = ceil_div(p.T * p.top_k + static_cast<int64_t>(p.E) * (kRowBlock - 1), kTM) + p.E;
+    const int64_t total = max_mtiles * ntiles_n;
     const unsigned grid = static_cast<unsigned>(round_up(total, kXcds));
     if (grid == 0) return 0;
+    constexpr int lds_bytes = kLdsBytes + kTouchBytes;
     // Opt in to more than 64 KB of dynamic LDS once per device.  The flags only cache an
     // idempotent runtime call; a race between threads at worst repeats it.
     static bool attr_set[64] = {};
@@ -237,17 +341,18 @@ int launch_gemm_tile(const MoeProblem& p, int mode, hipStream_t s) {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev]) {
         hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_kernel<1>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_kernel<2>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e1 != hipSuccess) return static_cast<int>(e1);
         if (e2 != hipSuccess) return static_cast<int>(e2);
         attr_set[dev] = true;
     }
     if (mode == 1)
-        hipLaunchKernelGGL(gemm_tile_kernel<1>, dim3(grid), dim3(kThreads), kLdsBytes, s, p, ntiles_n);
+        hipLaunchKernelGGL(gemm_tile_kernel<1>, dim3(grid, 1), dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, p.H);
     else
-        hipLaunchKernelGGL(gemm_tile_kernel<2>, dim3(grid), dim3(kThreads), kLdsBytes, s, p, ntiles_n);
+        hipLaunchKernelGGL(gemm_tile_kernel<2>, dim3(grid, static_cast<unsigned>(p.ksplit)), dim3(kThreads), lds_bytes,
+                           s, p, seg_begin, ntiles_n, p.I / p.ksplit);
     return launch_status();
 }
 

@@ -63,7 +63,7 @@ def test_workspace_layout_is_consistent():
                     (64, 256, 512), (4096, 6144, 16384)]:
         L = _lib.workspace_layout(T, H, I, 8, 2)
         assert lib.em_moe_workspace_bytes(T, H, I, 8, 2) == L.total_bytes
-        assert L.block_size == (16 if T <= 64 else 64 if T < 1024 else 256)
+        assert L.block_size == (16 if T <= 64 else 32)    # 32: the tiled kernel's fragment height
         assert L.sorted_len % L.block_size == 0 and L.sorted_len >= T * 2 + 8 * (L.block_size - 1)
         assert L.expert_ids_len * L.block_size == L.sorted_len
         offs = [L.topk_weights_off, L.topk_ids_off, L.sorted_ids_off, L.expert_ids_off, L.post_pad_off,
