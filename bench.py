@@ -39,6 +39,8 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=64, help="batch size T of the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
+    ap.add_argument("--shape", choices=["8x7b", "8x22b"], default="8x7b",
+                    help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
     ap.add_argument("--accurate", action="store_true",
                     help="run the layer with EM_FLAG_ACCURATE (bf16 hi+lo activations through the w2 GEMM)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -182,7 +184,10 @@ def calibrate_copy(torch, dev):
 
 
 def main():
+    global H, I
     args = parse_args()
+    if args.shape == "8x22b":
+        H, I = 6144, 16384
     if args.gpus != 1:
         print("bench.py measures one GPU: all experts are resident on a single MI355X and the layer uses "
               "no collectives; run with --gpus 1", file=sys.stderr)
@@ -220,22 +225,22 @@ def main():
 
     table = []
     if not args.no_table:
-        for t in (1, 8, 32, 256):
+        for t in ((1, 8, 32, 64, 256) if args.shape == "8x7b" else (1, 64)):
             if t != T:
                 table.append(measure(torch, t, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2)))
-        for lgk in ("normal", "zipf", "two_experts"):
-            r = measure(torch, 8192, w13, w2, 10, 3, logits=lgk)
+        for lgk in (("normal", "zipf", "two_experts") if args.shape == "8x7b" else ("normal",)):
+            r = measure(torch, 8192 if args.shape == "8x7b" else 4096, w13, w2, 10, 3, logits=lgk)
             r["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
             table.append(r)
     for r in [head] + table:
         r["hbm_frac"] = r["hbm_gbs"] / HBM_PEAK_GBS
 
     result = {
-        "metric": "Mixtral-8x7B MoE layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s",
+        "metric": f"Mixtral-{args.shape.upper().replace('X', 'x')} MoE layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"Mixtral-8x7B MoE layer decode T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
+        "config": {"workload": f"Mixtral-{args.shape} MoE layer T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
                                f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
                    "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate)},
         "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
