@@ -1,6 +1,6 @@
 // Shape-generic grouped expert GEMM on bf16 MFMA (v_mfma_f32_16x16x32_bf16).
 // This is the always-correct path: any H, I that are multiples of 8, any
-// sorted-block size in {16, 64}.  The tuned decode / prefill kernels replace it
+// sorted-block size in {16, 32} or a multiple of 64.  The tuned decode / prefill kernels replace it
 // for the shapes they support.
 //
 //   MODE 1  act[p, j] = bf16( silu(x[tok(p)] . w13[e, j]) * (x[tok(p)] . w13[e, I + j]) )
@@ -214,24 +214,24 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 }  // namespace
 
 int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s) {
-    if (p.block != 16 && p.block % 64 != 0) return EM_ERR_UNSUPPORTED;  // one 64-row tile never spans experts
-    const int tile_rows = (p.block == 16) ? 16 : 64;
+    // one row tile never spans experts: tile height = the sort block (16 or 32) or 64 for larger blocks
+    if (p.block != 16 && p.block != 32 && p.block % 64 != 0) return EM_ERR_UNSUPPORTED;
+    const int tile_rows = (p.block < 64) ? p.block : 64;
     const unsigned mblocks = static_cast<unsigned>(p.sorted_len / tile_rows);
     if (mblocks == 0) return 0;
     const dim3 blk(kThreads);
-    if (mode == 1) {
-        const dim3 grid(static_cast<unsigned>(ceil_div(p.I, kBR / 2)), mblocks, 1);
-        if (p.block == 16)
-            hipLaunchKernelGGL((gemm_generic_kernel<1, 1>), grid, blk, 0, s, p);
-        else
-            hipLaunchKernelGGL((gemm_generic_kernel<1, 4>), grid, blk, 0, s, p);
-    } else {
-        const dim3 grid(static_cast<unsigned>(ceil_div(p.H, kBR)), mblocks, static_cast<unsigned>(p.ksplit));
-        if (p.block == 16)
-            hipLaunchKernelGGL((gemm_generic_kernel<2, 1>), grid, blk, 0, s, p);
-        else
-            hipLaunchKernelGGL((gemm_generic_kernel<2, 4>), grid, blk, 0, s, p);
-    }
+    const dim3 grid = (mode == 1) ? dim3(static_cast<unsigned>(ceil_div(p.I, kBR / 2)), mblocks, 1)
+                                  : dim3(static_cast<unsigned>(ceil_div(p.H, kBR)), mblocks,
+                                         static_cast<unsigned>(p.ksplit));
+#define EM_LAUNCH_GENERIC(MODE)                                                             \
+    do {                                                                                    \
+        if (tile_rows == 16) hipLaunchKernelGGL((gemm_generic_kernel<MODE, 1>), grid, blk, 0, s, p);      \
+        else if (tile_rows == 32) hipLaunchKernelGGL((gemm_generic_kernel<MODE, 2>), grid, blk, 0, s, p); \
+        else hipLaunchKernelGGL((gemm_generic_kernel<MODE, 4>), grid, blk, 0, s, p);                      \
+    } while (0)
+    if (mode == 1) EM_LAUNCH_GENERIC(1);
+    else EM_LAUNCH_GENERIC(2);
+#undef EM_LAUNCH_GENERIC
     return launch_status();
 }
 

@@ -24,7 +24,7 @@ import numpy as np
 import pytest
 import torch
 
-from electrock_infer_amd import FusedMoE, fused_experts, moe_align_block_size
+from electrock_infer_amd import FusedMoE, _lib, fused_experts, moe_align_block_size
 from electrock_infer_amd.layers.moe.fused_moe import get_workspace
 from oracle import c_oracle, moe_oracle as O
 from tests.gpu_util import DEV, announce, error_stats, gpu_inputs, oracle_rows
@@ -236,3 +236,59 @@ def test_unsupported_inputs_raise():
         fused_experts(xb, w13.to(torch.bfloat16)[:, :, :128].contiguous(), w2.to(torch.bfloat16),
                       torch.zeros(4, 8, device=DEV), 2)
     assert fused_experts(xb[:0], w13.to(torch.bfloat16), w2.to(torch.bfloat16), torch.zeros(0, 8, device=DEV), 2).shape == (0, 256)
+
+
+# ---- shapes and routings that exercise every tile case of the GEMM kernels on a layer the oracle runs in full ----
+MID = dict(H=512, I=1024)
+
+
+def mid_inputs(T, routing, seed):
+    x, lg, w13, w2 = O.make_inputs(T, MID["H"], MID["I"], seed=seed, logits=routing if routing != "one_expert" else "normal")
+    if routing == "one_expert":
+        lg = lg.float()
+        lg[:, 3] += 30.0      # expert 3 takes every token's first slot; the second slot spreads over the rest
+        lg = lg.to(torch.bfloat16)
+    return x, lg, w13, w2
+
+
+@pytest.mark.parametrize("routing", ["normal", "zipf", "two_experts", "one_expert"])
+@pytest.mark.parametrize("T", [65, 96, 300, 513, 777, 1500, 4100])
+def test_layer_mid_shape_all_tile_cases(T, routing):
+    """T just above the streaming limit, around the split-K switch (512), experts with 0, 1 and several
+    256-row tiles, last tiles of every height; tuned kernels and the generic kernel against the oracle."""
+    announce(f"layer mid shape T={T} routing={routing}")
+    x, lg, w13, w2 = mid_inputs(T, routing, seed=T)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out_f32, out_bf16 = run_both(xd, lgd, w13d, w2d)
+    out_acc = run_accurate(xd, lgd, w13d, w2d)
+    check_routing(get_workspace(DEV, T, MID["H"], MID["I"], 8, 2), lg.float(), T)
+    check_outputs(f"mid_T{T}_{routing}", out_f32.cpu(), out_bf16.cpu(), ref, out_acc.cpu())
+    gen_f32, gen_bf16 = run_both(xd, lgd, w13d, w2d, flags=_lib.FLAG_FORCE_GENERIC)
+    check_outputs(f"mid_T{T}_{routing}_generic", gen_f32.cpu(), gen_bf16.cpu(), ref)
+
+
+@pytest.mark.parametrize("T", [1, 7, 33, 64])
+@pytest.mark.parametrize("routing", ["normal", "two_experts", "one_expert"])
+def test_layer_mid_shape_decode_cases(T, routing):
+    """Streaming kernel: experts with no tokens, with more than two 16-row fragments (second pass), generic cross-check."""
+    announce(f"layer mid shape decode T={T} routing={routing}")
+    x, lg, w13, w2 = mid_inputs(T, routing, seed=100 + T)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out_f32, out_bf16 = run_both(xd, lgd, w13d, w2d)
+    out_acc = run_accurate(xd, lgd, w13d, w2d)
+    check_routing(get_workspace(DEV, T, MID["H"], MID["I"], 8, 2), lg.float(), T)
+    check_outputs(f"mid_dec_T{T}_{routing}", out_f32.cpu(), out_bf16.cpu(), ref, out_acc.cpu())
+    gen_f32, gen_bf16 = run_both(xd, lgd, w13d, w2d, flags=_lib.FLAG_FORCE_GENERIC)
+    check_outputs(f"mid_dec_T{T}_{routing}_generic", gen_f32.cpu(), gen_bf16.cpu(), ref)
+
+
+def test_layer_shape_only_the_generic_kernel_supports():
+    """H and I that are multiples of 8 but fit neither tuned kernel."""
+    announce("layer odd shape H=136 I=200")
+    for T in (5, 70, 300):
+        x, lg, w13, w2 = O.make_inputs(T, 136, 200, seed=T)
+        ref = O.moe_layer_fp32(x, lg, w13, w2)
+        out_f32, out_bf16 = run_both(*(t.to(DEV) for t in (x, lg, w13, w2)))
+        check_outputs(f"odd_T{T}", out_f32.cpu(), out_bf16.cpu(), ref)
