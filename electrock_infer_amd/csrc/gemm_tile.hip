@@ -282,35 +282,74 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     if (nmi == 4) main_loop(std::true_type{});
     else main_loop(std::false_type{});
 
-    // ---- epilogue: element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 ----
+    // ---- epilogue.  Element v of lane l of a 32x32 accumulator sits at row 8*(v/4) + 4*(l/32) + v%4,
+    // column l%32: one column per lane.  Results are turned through LDS (free after the last stage) so
+    // that global stores are 16 bytes per lane on full 128-byte lines.
+    block_barrier();  // every wave has read its last operands: the stage buffers can be reused
     if (MODE == 1) {
-        const int j = nt * 128 + wn * 32 + r32;
+        // act tile [256 rows][128 columns] bf16, row pitch 272 B
+        constexpr int kPitchC = 128 * 2 + 16;
+        auto store_tile = [&](bool low_part) {
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-            if (mi >= nmi) break;
+            for (int mi = 0; mi < 4; ++mi) {
+                if (mi >= nmi) break;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
-                const float g = acc[mi][0][v];
-                const float u = acc[mi][1][v];
-                const float sg = g / (1.0f + __expf(-g));
-                store_act(p, (m0 + row) * static_cast<int64_t>(p.I) + j, sg * u);
+                for (int v = 0; v < 16; ++v) {
+                    const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
+                    const float g = acc[mi][0][v];
+                    const float u = acc[mi][1][v];
+                    const float val = g / (1.0f + __expf(-g)) * u;
+                    uint16_t bits = f32_to_bf16_bits(val);
+                    if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
+                    *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + r32) * 2) = bits;
+                }
             }
+            __syncthreads();
+            uint16_t* dst = low_part ? p.act_lo : p.act;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = tid + i * kThreads;  // 16-byte piece c of the tile: row c/16, columns (c%16)*8..+8
+                const int row = c >> 4;
+                if (row < valid)
+                    *reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + nt * 128 + (c & 15) * 8) =
+                        *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + (c & 15) * 16);
+            }
+        };
+        store_tile(false);
+        if (p.act_lo != nullptr) {
+            __syncthreads();
+            store_tile(true);
         }
     } else {
-        float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H;
+        // slots of the tile's rows -> LDS; then per wave and 32-row fragment a private [32][64] fp32 tile, pitch 272 B
+        constexpr int kPitchY = 64 * 4 + 16;
+        int32_t* slots = reinterpret_cast<int32_t*>(smem);
+        uint8_t* ytile = smem + 1024 + wave * (32 * kPitchY);
+        if (tid < kTM) slots[tid] = (tid < valid) ? p.sorted_ids[m0 + tid] : -1;
+        __syncthreads();
+        float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             if (mi >= nmi) break;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
-                const int slot = p.sorted_ids[m0 + row];
-                if (slot < 0) continue;
-                float* yrow = ybase + static_cast<int64_t>(slot) * p.H + nt * kTN + wn * 64 + r32;
-                yrow[0] = p.y_accumulate ? yrow[0] + acc[mi][0][v] : acc[mi][0][v];
-                yrow[32] = p.y_accumulate ? yrow[32] + acc[mi][1][v] : acc[mi][1][v];
+                const int row = 8 * (v >> 2) + 4 * kh + (v & 3);
+                *reinterpret_cast<float*>(ytile + row * kPitchY + r32 * 4) = acc[mi][0][v];
+                *reinterpret_cast<float*>(ytile + row * kPitchY + (32 + r32) * 4) = acc[mi][1][v];
             }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                const int row = it * 4 + (lane >> 4);
+                const int slot = slots[wm * 128 + mi * 32 + row];
+                f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane & 15) * 16);
+                if (slot >= 0) {
+                    f32x4_t* dst = reinterpret_cast<f32x4_t*>(ybase + static_cast<int64_t>(slot) * p.H + (lane & 15) * 4);
+                    if (p.y_accumulate) val += *dst;
+                    *dst = val;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
         }
     }
 }
