@@ -15,6 +15,11 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 // Up to this many tokens the weight-streaming GEMM runs (16-row sorted blocks, a
 // couple of MFMA fragments per expert); above it the tiled kernels take over.
 constexpr int64_t kStreamMaxT = 64;
+// Tile height of the tiled kernels by batch size (8 experts, top-2: T/4 rows per expert on
+// average): 64-row tiles while most experts fit one of them, 128-row tiles likewise, then the
+// 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 448 tokens.
+constexpr int64_t kTile64MaxT = 192;
+constexpr int64_t kTile128MaxT = 448;
 
 // Rows per sorted block, the counterpart of _get_moe_config (fused_moe.py:327-339):
 // 16 (one MFMA fragment) for the streaming kernel, 32 for the tiled kernel, which cuts
@@ -23,11 +28,11 @@ inline int choose_block(int64_t T, int H, int I) {
     if (T <= kStreamMaxT) return 16;
     return tile_shape_ok(H, I) ? tile_row_block() : 64;
 }
-// Split of the w2 reduction (K = I) across workgroups for small batches, where
-// (row tiles) x (column tiles) alone would leave most CUs idle.
+// Split of the w2 reduction (K = I) across workgroups: (row tiles) x (H / 256 column tiles)
+// alone leaves CUs idle for small batches and ends in a ragged last round for large ones.
 inline int choose_ksplit(int64_t T, int H, int I) {
     if (T > kStreamMaxT) {
-        const int want = T <= 512 ? 4 : 1;
+        const int want = 2;  // two K slices measure fastest from 128 to 8192 tokens
         if (!tile_shape_ok(H, I)) return want;
         for (int ks = want; ks >= 1; --ks)  // the tiled kernel needs I / ksplit to be a multiple of 64
             if (I % (ks * 64) == 0) return ks;
@@ -199,22 +204,27 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
     }
     const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
     const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T > kStreamMaxT && tile_supported(p);
+    auto tile_gemm = [&](const MoeProblem& q, int mode) {
+        if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
+        if (T <= kTile128MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
+        return launch_gemm_tile(q, seg_begin, mode, s);
+    };
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
         rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s)
-             : use_tile ? launch_gemm_tile(p, seg_begin, 1, s) : launch_gemm_generic(p, 1, s);
+             : use_tile ? tile_gemm(p, 1) : launch_gemm_generic(p, 1, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
         if (use_stream) {
             rc = launch_gemm_stream(p, seg_begin, 2, s);  // multiplies act and act_lo in one pass
         } else {
-            rc = use_tile ? launch_gemm_tile(p, seg_begin, 2, s) : launch_gemm_generic(p, 2, s);
+            rc = use_tile ? tile_gemm(p, 2) : launch_gemm_generic(p, 2, s);
             if (rc == 0 && accurate) {  // second pass: y += act_lo . w2
                 MoeProblem lo = p;
                 lo.act = p.act_lo;
                 lo.act_lo = nullptr;
                 lo.y_accumulate = 1;
-                rc = use_tile ? launch_gemm_tile(lo, seg_begin, 2, s) : launch_gemm_generic(lo, 2, s);
+                rc = use_tile ? tile_gemm(lo, 2) : launch_gemm_generic(lo, 2, s);
             }
         }
         if (rc != 0) return rc;

@@ -34,6 +34,7 @@
 //              tiles, ordered 4 row tiles x all column tiles, which lets the 32
 //              CUs of an XCD share A and B tiles through their own L2.
 #include "common.h"
+#include "lds_copy.h"
 #include <type_traits>
 
 namespace em {
@@ -52,29 +53,6 @@ constexpr int kGroupM = 4;
 constexpr int kXcds = 8;
 constexpr int kDmaPerStage = kStageBytes / (kThreads * 16);  // 8 per thread
 constexpr int kDmaHalf = kDmaPerStage / 2;                   // first half A rows, second half B rows
-
-// M0 is a reserved register that the compiler never keeps live values in here (the
-// kernel has no dynamically indexed register arrays); naming it as a clobber documents
-// the write and only triggers an advisory warning.
-#pragma clang diagnostic ignored "-Winline-asm"
-
-// One wave copies 64 x 16 B from per-lane global addresses to 1 KB of LDS starting at
-// the wave-uniform byte address `lds_addr`.  The compiler does not see the LDS write:
-// every consumer sits behind wait_dma<>() + block_barrier().
-__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
-}
-template <int N>
-__device__ __forceinline__ void wait_dma() {  // at most N of this wave's copies still in flight
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
-}
-// Same for one dword per lane (256 B of LDS per wave): used only to pull lines into L2.
-__device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
-                 :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
-}
-__device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 template <int MODE>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
