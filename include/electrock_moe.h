@@ -143,8 +143,8 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  * EM_FLAG_ACCURATE keeps the SiLU*mul activations as a bf16 pair (value, rounding
  * residual) and multiplies both with w2, which removes the one rounding the bf16 MFMA
  * of the w2 GEMM otherwise needs; together with EM_FLAG_OUT_F32 the result is within
- * fp32 accumulation error of the fp32 definition.  Free for T <= 64 (the layer is
- * HBM-bound there), one extra w2 pass otherwise.
+ * fp32 accumulation error of the fp32 definition.  Costs ~14 % at T = 64 (no extra
+ * weight traffic, more operand loads) and one extra w2 pass for T > 64.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.
