@@ -2,7 +2,8 @@
 // per expert), where the layer moves from HBM-bound to bound by the bf16 MFMA rate.
 //
 //   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile of up to 256 sorted rows x 256
-//              weight rows; K in steps of 64 through two 64 KB LDS stages
+//              weight rows; K in steps of 64; LDS (all 160 KB) holds a ring of two 32 KB
+//              slots of token rows (A) and a ring of three 32 KB slots of weight rows (B)
 //   tiles      the sort pads experts to 32 rows only; every expert is cut into 256-row
 //              tiles and its last tile is as high as the rows that are left (a multiple
 //              of 32).  A wave multiplies only the 32-row fragments that exist, so a
@@ -11,14 +12,15 @@
 //              segment starts (at most 64 scalar loads).
 //   loads      global -> LDS directly (global_load_lds_dwordx4), no registers in
 //              between; eight lanes fetch one full 128-byte line of a row (measured
-//              L2 -> CU feed: ~23 TB/s with 128 B per row against ~16 TB/s with 64 B);
-//              the copy of stage k+1 runs while stage k is multiplied; completion is
-//              tracked by hand with s_waitcnt vmcnt + one s_barrier per stage
-//   prefetch   a stage only completes when its slowest line has arrived, and the first
-//              workgroup of an XCD to ask for a line pays HBM latency; so every
-//              workgroup also touches (one dword per line, into a dummy LDS area) its
-//              share of the lines that the workgroups sharing its A and B tiles will
-//              need six stages later, which turns those misses into L2 hits
+//              L2 -> CU feed: ~26 TB/s with 128 B per row against ~17 TB/s with 64 B).
+//              Weight rows stream from HBM and are requested two K steps before their
+//              use, token rows (L2 / memory-side cache hits) one step before; with a
+//              single stage in flight the slowest line of a stage, at HBM latency, sat
+//              on the critical path of every step.  Completion is tracked by hand with
+//              s_waitcnt vmcnt + one s_barrier per step.
+//   issue      the eight copy instructions of a wave are issued one by one between the
+//              eight MFMAs that follow the barrier: issued back to back (by both waves of
+//              a SIMD at once) they left the matrix pipe idle for a fifth of every step
 //   LDS        rows are 128 B; the 16-byte pieces of every 2-row group are XOR-
 //              swizzled so that the 16 lanes of a b128 operand read hit 16 bank groups
 //   wave       128 x 64 sub-tile = 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (the
@@ -42,17 +44,15 @@ namespace {
 
 constexpr int kTM = 256, kTN = 256, kTK = 64;
 constexpr int kThreads = 512;
-constexpr int kStages = 2;
-constexpr int kRegionBytes = kTM * kTK * 2;          // 32 KB: A rows, then 32 KB of B rows
-constexpr int kStageBytes = 2 * kRegionBytes;        // 64 KB
-constexpr int kLdsBytes = kStages * kStageBytes;     // 128 KB
-constexpr int kTouchBytes = 8 * 256;                 // dummy landing area of the L2 touches
-constexpr int kTouchAhead = 6;                       // stages between a touch and its use
+constexpr int kSlotBytes = kTM * kTK * 2;            // 32 KB: 256 rows x 64 K of one operand
+constexpr int kSlotsA = 2, kSlotsB = 3;
+constexpr int kOffB = kSlotsA * kSlotBytes;          // B ring behind the A ring
+constexpr int kLdsBytes = (kSlotsA + kSlotsB) * kSlotBytes;  // 160 KB
 constexpr int kRowBlock = 32;                        // sort padding this kernel needs
 constexpr int kGroupM = 4;
 constexpr int kXcds = 8;
-constexpr int kDmaPerStage = kStageBytes / (kThreads * 16);  // 8 per thread
-constexpr int kDmaHalf = kDmaPerStage / 2;                   // first half A rows, second half B rows
+constexpr int kDmaHalf = kSlotBytes / (kThreads * 16);  // 4 copies per thread and operand slot
+constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, second half B rows
 
 template <int MODE>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
@@ -97,10 +97,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     // ---- copy plan: copy n of a stage lands at region n / 4, byte (n % 4) * 8 KB + wave * 1 KB + lane * 16.
     // Byte o of a region holds piece q ^ (u & 7) of 2-row group u = o / 256, q = (row & 1) * 8 + piece.
     // One copy covers 8 whole rows; copies of A rows beyond `valid` are skipped.
-    const uint16_t* src[kDmaPerStage];
+    // Addresses are a wave-uniform base per operand plus a 32-bit byte offset per lane.
+    uint32_t voff[kDmaPerStage];
     bool live[kDmaPerStage];
     const uint16_t* wbase = (MODE == 1) ? p.w13 + static_cast<int64_t>(expert) * 2 * p.I * p.H
                                         : p.w2 + static_cast<int64_t>(expert) * p.H * p.I;
+    const uint8_t* base_a = reinterpret_cast<const uint8_t*>(((MODE == 1) ? p.x : p.act + m0 * static_cast<int64_t>(p.I)) + k_begin);
+    const uint8_t* base_b = reinterpret_cast<const uint8_t*>(wbase + k_begin);
 #pragma unroll
     for (int n = 0; n < kDmaPerStage; ++n) {
         const int o = (n % kDmaHalf) * 8192 + wave * 1024 + lane * 16;
@@ -114,60 +117,40 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             if (MODE == 1) {
                 const int slot = p.sorted_ids[m0 + rr];
                 const int tok = (slot >= 0) ? slot / p.top_k : 0;  // pad rows multiply token 0; never stored
-                src[n] = p.x + static_cast<int64_t>(tok) * p.H + k_begin + piece * 8;
+                voff[n] = static_cast<uint32_t>(tok) * static_cast<uint32_t>(p.H * 2) + piece * 16;
             } else {
-                src[n] = p.act + (m0 + rr) * static_cast<int64_t>(p.I) + k_begin + piece * 8;
+                voff[n] = static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.I * 2) + piece * 16;
             }
         } else {
             live[n] = true;
-            int64_t grow;
+            uint32_t grow;
             if (MODE == 1)  // LDS row r of the B tile: wave column r/64, gate (0) or up (1) half, j offset r%32
-                grow = static_cast<int64_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31);
+                grow = static_cast<uint32_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31);
             else
-                grow = static_cast<int64_t>(nt) * kTN + r;
-            src[n] = wbase + grow * K + k_begin + piece * 8;
+                grow = static_cast<uint32_t>(nt) * kTN + r;
+            voff[n] = grow * static_cast<uint32_t>(K * 2) + piece * 16;
         }
     }
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
-    auto issue = [&](int stage_k, int buf) {  // stage_k: K step index, buf: ring slot
-        const int k0 = stage_k * kTK;
-#pragma unroll
-        for (int n = 0; n < kDmaPerStage; ++n)
-            if (live[n])
-                dma16(src[n] + k0, dma_base + buf * kStageBytes + (n / kDmaHalf) * kRegionBytes + (n % kDmaHalf) * 8192);
-    };
-
-    // ---- L2 touch plan: line id = wave * 64 + lane, 0..255 = A rows, 256..511 = B rows.  The up to 8 column
-    // tiles that run next to this one share its A tile and the 4 row tiles of its group share its B tile, so
-    // this workgroup touches every 8th A line and every 4th B line; other lanes repeat line 0 (coalesced away).
-    // Every wave issues exactly one touch per stage, which keeps the vmcnt bookkeeping uniform.
-    const uint16_t* touch_src;
-    {
-        const int tl = wave * 64 + lane;
-        const int trow = tl & 255;
-        if (tl < 256) {
-            const bool mine = (trow & 7) == (nt & 7) && trow < valid;
-            const int rr = mine ? trow : 0;
-            if (MODE == 1) {
-                const int slot = p.sorted_ids[m0 + rr];
-                touch_src = p.x + static_cast<int64_t>(slot >= 0 ? slot / p.top_k : 0) * p.H + k_begin;
-            } else {
-                touch_src = p.act + (m0 + rr) * static_cast<int64_t>(p.I) + k_begin;
-            }
-        } else {
-            const bool mine = (trow & 3) == m_in_group;
-            const int r = mine ? trow : 0;
-            const int64_t grow = (MODE == 1)
-                                     ? static_cast<int64_t>((r >> 5) & 1) * p.I + nt * 128 + (r >> 6) * 32 + (r & 31)
-                                     : static_cast<int64_t>(nt) * kTN + r;
-            touch_src = wbase + grow * K + k_begin;
-        }
-    }
-    const uint32_t touch_dst = __builtin_amdgcn_readfirstlane(lds0 + kLdsBytes + wave * 256);
     const int nk = kslice / kTK;
-    auto touch = [&](int stage_k) {
-        dma4(touch_src + (stage_k < nk ? stage_k : nk - 1) * kTK, touch_dst);
+    // copy n (0..3) of the token rows / weight rows of K step stage_k
+    auto copy_a = [&](int n, int stage_k) {
+        dma16(voff[n], base_a + static_cast<int64_t>(stage_k) * (kTK * 2),
+              dma_base + (stage_k & 1) * kSlotBytes + n * 8192);
+    };
+    auto copy_b = [&](int n, int stage_k, int slot) {
+        dma16(voff[kDmaHalf + n], base_b + static_cast<int64_t>(stage_k) * (kTK * 2),
+              dma_base + kOffB + slot * kSlotBytes + n * 8192);
+    };
+    auto issue_a = [&](int stage_k) {
+#pragma unroll
+        for (int n = 0; n < kDmaHalf; ++n)
+            if (live[n]) copy_a(n, stage_k);
+    };
+    auto issue_b = [&](int stage_k, int slot) {
+#pragma unroll
+        for (int n = 0; n < kDmaHalf; ++n) copy_b(n, stage_k, slot);
     };
 
     f32x16_t acc[4][2];
@@ -188,7 +171,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         const int piece = (ks * 2 + kh) ^ sw;
         const int ra = wm * 128 + r32, rb = wn * 64 + r32;
         a_off[ks] = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
-        b_off[ks] = kRegionBytes + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
+        b_off[ks] = kOffB + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
     }
     // 32-row fragments of this wave that hold rows of the tile (wave-uniform)
     int nmi = (valid - wm * 128 + 31) / 32;
@@ -196,69 +179,117 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     nmi = __builtin_amdgcn_readfirstlane(nmi);
 
     bf16x8_t fa[2][4], fb[2][2];
-    // FULL: all four fragments exist (the common case) -> fixed instruction mix with scheduling hints
-    auto main_loop = [&](auto full_tag) {
+    // operand fragments of 16-wide K step ks of K step stage_k (weight rows in ring slot bslot) -> register set `set`
+    auto read_frags = [&](int stage_k, int bslot, int ks, int set, auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;
-        auto read_frags = [&](const uint8_t* s, int ks, int set) {
+        const uint8_t* sa = smem + (stage_k & 1) * kSlotBytes;
+        const uint8_t* sb = smem + bslot * kSlotBytes;
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
-                if (FULL || mi < nmi) fa[set][mi] = *reinterpret_cast<const bf16x8_t*>(s + a_off[ks] + mi * 4096);
+        for (int mi = 0; mi < 4; ++mi)
+            if (FULL || mi < nmi) fa[set][mi] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[ks] + mi * 4096);
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const bf16x8_t*>(s + b_off[ks] + ni * 4096);
-        };
-        auto multiply = [&](int set) {
-#pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
-                if (FULL || mi < nmi) {
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
-                }
-            if (FULL) {  // scheduling hint: one LDS read after each of the first six MFMAs, then the last two
-#pragma unroll
-                for (int i = 0; i < 6; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            }
-        };
-        const bool work = FULL || nmi > 0;  // waves without rows still copy, touch and meet the barriers
-        issue(0, 0);
-        touch(1);
-        wait_dma<1>();  // everything but the touch
-        block_barrier();
-        if (1 < nk) issue(1, 1);
-        touch(2);
-        if (work) read_frags(smem, 0, 0);
-        for (int kt = 0; kt + 1 < nk; ++kt) {
-            const uint8_t* s = smem + (kt & 1) * kStageBytes;
-            if (work) {
-                read_frags(s, 1, 1); multiply(0);
-                read_frags(s, 2, 0); multiply(1);
-                read_frags(s, 3, 1); multiply(0);
-            }
-            wait_dma<1>();                                      // this wave's part of stage kt+1 is in LDS
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of stage kt are in registers
-            block_barrier();                                    // ... and so are everyone else's
-            if (kt + 2 < nk) issue(kt + 2, kt & 1);             // stage kt's buffer is free again
-            touch(kt + 2 + kTouchAhead);
-            if (work) {
-                read_frags(smem + ((kt + 1) & 1) * kStageBytes, 0, 0);
-                multiply(1);
-            }
-        }
-        if (work) {  // last stage: nothing left to copy
-            const uint8_t* s = smem + ((nk - 1) & 1) * kStageBytes;
-            read_frags(s, 1, 1); multiply(0);
-            read_frags(s, 2, 0); multiply(1);
-            read_frags(s, 3, 1); multiply(0);
-            multiply(1);
-        }
-        wait_dma<0>();  // the last touches must not outlive the workgroup's LDS
+        for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[ks] + ni * 4096);
     };
-    if (nmi == 4) main_loop(std::true_type{});
-    else main_loop(std::false_type{});
+    auto multiply = [&](int set, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+            if (FULL || mi < nmi) {
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
+            }
+        if (FULL) {  // scheduling hint: one LDS read after each of the first six MFMAs, then the last two
+#pragma unroll
+            for (int i = 0; i < 6; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+    };
+    auto next_slot = [](int slot) { return slot == kSlotsB - 1 ? 0 : slot + 1; };
+
+    // Copies are queued per wave in the order  A(0) B(0) B(1) | A(1) B(2) | A(2) B(3) | ...  so that at the end
+    // of step kt everything but the newest four copies (B(kt+2)) has to be in LDS: vmcnt(4), vmcnt(0) at the end.
+    issue_a(0);
+    issue_b(0, 0);
+    if (1 < nk) {
+        issue_b(1, 1);
+        wait_dma<kDmaHalf>();
+    } else {
+        wait_dma<0>();
+    }
+    block_barrier();
+    if (1 < nk) issue_a(1);
+    if (2 < nk) issue_b(2, 2);
+    int bs = 0;  // ring slot of the weight rows of step kt
+    if (nmi == 4) {
+        // All four fragments exist (the common case): fixed instruction mix.  After the barrier that ends step
+        // kt, the eight MFMAs of its last 16-wide K step alternate with the copies of A(kt+2) and B(kt+3) (the
+        // slots step kt has just freed) and with the first operand reads of step kt+1.
+        const std::true_type full;
+        read_frags(0, 0, 0, 0, full);
+        auto step = [&](int kt, auto copy_a_tag, auto copy_b_tag) {
+            constexpr bool CA = decltype(copy_a_tag)::value, CB = decltype(copy_b_tag)::value;
+            read_frags(kt, bs, 1, 1, full); multiply(0, full);
+            read_frags(kt, bs, 2, 0, full); multiply(1, full);
+            read_frags(kt, bs, 3, 1, full); multiply(0, full);
+            if (CA) wait_dma<kDmaHalf>(); else wait_dma<0>();   // this wave's parts of A(kt+1), B(kt+1) are in LDS
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of step kt are in registers
+            block_barrier();                                    // ... and so are everyone else's
+            __builtin_amdgcn_sched_barrier(0);
+            const int bn = next_slot(bs);
+            const uint8_t* sa = smem + ((kt + 1) & 1) * kSlotBytes;
+            const uint8_t* sb = smem + bn * kSlotBytes;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i >> 1], fb[1][i & 1], acc[i >> 1][i & 1], 0, 0, 0);
+                if (i < 4) { if (CA) copy_a(i, kt + 2); } else { if (CB) copy_b(i - 4, kt + 3, bs); }
+                if (i < 4) fa[0][i] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0] + i * 4096);
+                else if (i < 6) fb[0][i - 4] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0] + (i - 4) * 4096);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            bs = bn;
+        };
+        int kt = 0;
+        for (; kt + 3 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
+        for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::false_type{});
+        for (; kt + 1 < nk; ++kt) step(kt, std::false_type{}, std::false_type{});
+        read_frags(nk - 1, bs, 1, 1, full); multiply(0, full);
+        read_frags(nk - 1, bs, 2, 0, full); multiply(1, full);
+        read_frags(nk - 1, bs, 3, 1, full); multiply(0, full);
+        multiply(1, full);
+    } else {
+        // Short tile: a wave multiplies the fragments that exist; waves without rows still copy and meet the
+        // barriers.  Skipped copies of missing token rows do not change the counts: the newest four are B's.
+        const std::false_type part;
+        const bool work = nmi > 0;
+        if (work) read_frags(0, 0, 0, 0, part);
+        for (int kt = 0; kt + 1 < nk; ++kt) {
+            if (work) {
+                read_frags(kt, bs, 1, 1, part); multiply(0, part);
+                read_frags(kt, bs, 2, 0, part); multiply(1, part);
+                read_frags(kt, bs, 3, 1, part); multiply(0, part);
+            }
+            if (kt + 2 < nk) wait_dma<kDmaHalf>(); else wait_dma<0>();
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            block_barrier();
+            if (kt + 2 < nk) issue_a(kt + 2);
+            if (kt + 3 < nk) issue_b(kt + 3, bs);
+            bs = next_slot(bs);
+            if (work) {
+                read_frags(kt + 1, bs, 0, 0, part);
+                multiply(1, part);
+            }
+        }
+        if (work) {
+            read_frags(nk - 1, bs, 1, 1, part); multiply(0, part);
+            read_frags(nk - 1, bs, 2, 0, part); multiply(1, part);
+            read_frags(nk - 1, bs, 3, 1, part); multiply(0, part);
+            multiply(1, part);
+        }
+    }
 
     // ---- epilogue.  Element v of lane l of a 32x32 accumulator sits at row 8*(v/4) + 4*(l/32) + v%4,
     // column l%32: one column per lane.  Results are turned through LDS (free after the last stage) so
@@ -338,8 +369,11 @@ bool tile_shape_ok(int H, int I) { return H % kTN == 0 && I % 128 == 0 && H % kT
 int tile_row_block() { return kRowBlock; }
 
 bool tile_supported(const MoeProblem& p) {
+    // copy addresses are 32-bit byte offsets from x, from an expert's weights and from a tile of act
+    const int64_t lim = int64_t{1} << 32;
     return p.block == kRowBlock && tile_shape_ok(p.H, p.I) && p.T > 0 && p.ksplit >= 1 &&
-           p.I % (p.ksplit * kTK) == 0;
+           p.I % (p.ksplit * kTK) == 0 && p.T * p.H * 2 < lim && int64_t{4} * p.I * p.H < lim &&
+           int64_t{kTM} * p.I * 2 < lim;
 }
 
 int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s) {
@@ -350,7 +384,7 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     const int64_t total = max_mtiles * ntiles_n;
     const unsigned grid = static_cast<unsigned>(round_up(total, kXcds));
     if (grid == 0) return 0;
-    constexpr int lds_bytes = kLdsBytes + kTouchBytes;
+    constexpr int lds_bytes = kLdsBytes;
     // Opt in to more than 64 KB of dynamic LDS once per device.  The flags only cache an
     // idempotent runtime call; a race between threads at worst repeats it.
     static bool attr_set[64] = {};

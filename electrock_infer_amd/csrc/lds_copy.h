@@ -17,6 +17,12 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
+// Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit byte
+// offset per lane: half the address registers, and stepping through K is scalar arithmetic.
+__device__ __forceinline__ void dma16(uint32_t lane_offset, const void* uniform_base, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_offset), "s"(uniform_base), "s"(lds_addr) : "memory", "m0");
+}
 template <int N>
 __device__ __forceinline__ void wait_dma() {  // at most N of this wave's copies still in flight
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
