@@ -24,10 +24,14 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);  // NaN
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    const __bf16 b = static_cast<__bf16>(f);  // v_cvt_pk_bf16_f32: round to nearest even, NaN stays NaN
+    uint16_t h;
+    __builtin_memcpy(&h, &b, 2);
+    return h;
+}
+// SiLU(g) * u in fp32 for the fused GEMM epilogues; the reciprocal is the hardware's (1 ulp)
+__device__ __forceinline__ float silu_mul(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     _Float16 v;
@@ -44,7 +48,13 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return static_cast<uint32_t>(f32_to_bf16_bits(lo)) | (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    bf16x2_t v;
+    v[0] = static_cast<__bf16>(lo);
+    v[1] = static_cast<__bf16>(hi);
+    uint32_t w;
+    __builtin_memcpy(&w, &v, 4);
+    return w;
 }
 
 // Element traits for the three storage types the ops accept.

@@ -162,8 +162,7 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(MoeProblem p) {
                 for (int v = 0; v < 4; ++v) {
                     const float g = acc[f][0][v];
                     const float u = acc[f][1][v];
-                    const float s = g / (1.0f + __expf(-g));
-                    store_act(p, (m0 + f * 16 + kq * 4 + v) * static_cast<int64_t>(p.I) + j, s * u);
+                    store_act(p, (m0 + f * 16 + kq * 4 + v) * static_cast<int64_t>(p.I) + j, silu_mul(g, u));
                 }
         }
     } else {

@@ -191,9 +191,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
                     const f32x4_t u = total(f, 2 + wave);
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
-                        const float s = g[v] / (1.0f + __expf(-g[v]));
                         const int64_t row = seg + (f0 + f) * 16 + kq * 4 + v;
-                        store_act(p, row * p.I + j, s * u[v]);
+                        store_act(p, row * p.I + j, silu_mul(g[v], u[v]));
                     }
                 }
             }

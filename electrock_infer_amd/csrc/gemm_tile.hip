@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
                     const float g = acc[mi][0][v];
                     const float u = acc[mi][1][v];
-                    const float val = g / (1.0f + __expf(-g)) * u;
+                    const float val = silu_mul(g, u);
                     uint16_t bits = f32_to_bf16_bits(val);
                     if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
                     *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + r32) * 2) = bits;
