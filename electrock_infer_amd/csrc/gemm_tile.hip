@@ -31,10 +31,10 @@
 //              up rows I + j, so SiLU(g) * u is lane-local in the epilogue
 //   MODE 2     256 rows of w2[e], optionally one of `ksplit` K slices; fp32 partial rows
 //              are scattered to y[z, slot]
-//   order      workgroup ids are dealt to the 8 XCDs round-robin by the hardware;
-//              they are re-mapped so that each XCD walks one contiguous range of
-//              tiles, ordered 4 row tiles x all column tiles, which lets the 32
-//              CUs of an XCD share A and B tiles through their own L2.
+//   order      workgroup ids are dealt to the 8 XCDs round-robin by the hardware; each XCD
+//              takes an eighth of the column tiles of every expert and walks them expert by
+//              expert, column by column, row tile fastest, so that the 32 CUs of an XCD share
+//              weight and token tiles through their own L2 and weights leave HBM once.
 #include "common.h"
 #include "lds_copy.h"
 #include <type_traits>
@@ -62,25 +62,43 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     // ---- tile list: expert e owns ceil(rows_e / 256) row tiles ----
     int mtiles = 0;
     for (int e = 0; e < p.E; ++e) mtiles += (seg_begin[e + 1] - seg_begin[e] + kTM - 1) / kTM;
-    // ---- which tile: XCD-aware re-mapping over the ACTUAL number of row tiles ----
-    const int total = mtiles * ntiles_n;
-    const int per_xcd = (total + kXcds - 1) / kXcds;
-    const int xcd = blockIdx.x % kXcds;
-    const int local = blockIdx.x / kXcds;
-    const int logical = xcd * per_xcd + local;
-    if (local >= per_xcd || logical >= total) return;
-    const int group_sz = kGroupM * ntiles_n;
-    const int group = logical / group_sz;
-    const int in_group = logical - group * group_sz;
-    const int rows_in_group = (mtiles - group * kGroupM < kGroupM) ? mtiles - group * kGroupM : kGroupM;
-    const int m_in_group = in_group % rows_in_group;
-    const int nt = in_group / rows_in_group;
-    int mt = group * kGroupM + m_in_group;  // global row-tile index -> (expert, tile inside the expert)
-    int expert = 0;
-    for (; expert < p.E - 1; ++expert) {
-        const int t = (seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM;
-        if (mt < t) break;
-        mt -= t;
+    // ---- which tile.  Workgroup ids are dealt to the 8 XCDs round-robin by the hardware; XCD x takes the
+    // column tiles [x, x+1) * ntiles_n / 8 of every expert and walks them expert by expert, column by column,
+    // row tile fastest.  The CUs of an XCD then share a few weight tiles and all row tiles of the expert through
+    // their L2, every weight byte leaves HBM once, and the eight XCDs read the same token rows at the same time.
+    int nt, mt, expert = 0;
+    if (ntiles_n % kXcds == 0) {
+        const int cols = ntiles_n / kXcds;
+        const int xcd = blockIdx.x % kXcds;
+        int local = blockIdx.x / kXcds;
+        if (local >= mtiles * cols) return;
+        for (; expert < p.E - 1; ++expert) {
+            const int t = ((seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM) * cols;
+            if (local < t) break;
+            local -= t;
+        }
+        const int rows_e = (seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM;
+        nt = xcd * cols + local / rows_e;
+        mt = local % rows_e;
+    } else {
+        // column count not divisible: contiguous ranges of 4 row tiles x all column tiles per XCD
+        const int total = mtiles * ntiles_n;
+        const int per_xcd = (total + kXcds - 1) / kXcds;
+        const int xcd = blockIdx.x % kXcds;
+        const int local = blockIdx.x / kXcds;
+        const int logical = xcd * per_xcd + local;
+        if (local >= per_xcd || logical >= total) return;
+        const int group_sz = kGroupM * ntiles_n;
+        const int group = logical / group_sz;
+        const int in_group = logical - group * group_sz;
+        const int rows_in_group = (mtiles - group * kGroupM < kGroupM) ? mtiles - group * kGroupM : kGroupM;
+        nt = in_group / rows_in_group;
+        mt = group * kGroupM + in_group % rows_in_group;  // global row-tile index -> (expert, tile inside the expert)
+        for (; expert < p.E - 1; ++expert) {
+            const int t = (seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM;
+            if (mt < t) break;
+            mt -= t;
+        }
     }
     const int64_t m0 = seg_begin[expert] + static_cast<int64_t>(mt) * kTM;
     const int rows_left = seg_begin[expert + 1] - static_cast<int>(m0);
