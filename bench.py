@@ -43,14 +43,24 @@ def parse_args():
                     help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
     ap.add_argument("--accurate", action="store_true",
                     help="run the layer with EM_FLAG_ACCURATE (bf16 hi+lo activations through the w2 GEMM)")
+    ap.add_argument("--operands", choices=["gaussian", "zeros"], default="gaussian",
+                    help="values of x and the expert weights.  'zeros' is a diagnostic: the matrix pipes then draw "
+                         "little power and the same kernels run at the full shader clock, which separates the "
+                         "board's power limit from the kernels' own stalls; never the headline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three device copies of 1 GiB (a plain copy kernel of known size that the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by)")
     return ap.parse_args()
 
 
+OPERANDS = "gaussian"
+
+
 def make_weights(torch, dev):
     g = torch.Generator(device=dev).manual_seed(0)
+    if OPERANDS == "zeros":
+        return (torch.zeros(E, 2 * I, H, device=dev, dtype=torch.bfloat16),
+                torch.zeros(E, H, I, device=dev, dtype=torch.bfloat16))
     w13 = torch.empty(E, 2 * I, H, device=dev, dtype=torch.bfloat16)
     w2 = torch.empty(E, H, I, device=dev, dtype=torch.bfloat16)
     for e in range(E):
@@ -62,6 +72,8 @@ def make_weights(torch, dev):
 def make_batch(torch, dev, T, seed=0, logits="normal"):
     g = torch.Generator(device=dev).manual_seed(1000 + seed)
     x = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    if OPERANDS == "zeros":
+        x.zero_()
     lg = torch.randn(T, E, generator=g, device=dev, dtype=torch.float32)
     if logits == "zipf":
         ranks = torch.arange(1, E + 1, dtype=torch.float32) ** -1.2
@@ -184,8 +196,9 @@ def calibrate_copy(torch, dev):
 
 
 def main():
-    global H, I
+    global H, I, OPERANDS
     args = parse_args()
+    OPERANDS = args.operands
     if args.shape == "8x22b":
         H, I = 6144, 16384
     if args.gpus != 1:
@@ -239,7 +252,7 @@ def main():
         "metric": f"Mixtral-{args.shape.upper().replace('X', 'x')} MoE layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic" if args.operands == "gaussian" else "synthetic, all-zero x and weights (diagnostic)",
         "config": {"workload": f"Mixtral-{args.shape} MoE layer T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
                                f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
                    "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate)},
