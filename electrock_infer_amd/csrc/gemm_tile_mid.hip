@@ -113,7 +113,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_mid_kernel(MoeProblem p
         const int k0 = stage_k * kTK;
 #pragma unroll
         for (int n = 0; n < kCopies; ++n)
-            dma16(src[n] + k0, dma_base + buf * kStageBytes + (n < MI ? n * 8192 : kABytes + (n - MI) * 8192));
+            if (n < MI) dma16(src[n] + k0, dma_base + buf * kStageBytes + n * 8192);                             // token rows: shared
+            else dma16_stream(src[n] + k0, dma_base + buf * kStageBytes + kABytes + (n - MI) * 8192);   // weight rows: read once
     };
 
     f32x16_t acc[MI][2];

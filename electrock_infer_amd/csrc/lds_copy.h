@@ -17,6 +17,12 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
+// Same copy for data that no other workgroup reads again (weight rows streamed once): the non-temporal
+// hint keeps them from displacing reusable lines; plain reads of a stream top out ~15 % lower on this GPU.
+__device__ __forceinline__ void dma16_stream(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+                 :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
 // Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit byte
 // offset per lane: half the address registers, and stepping through K is scalar arithmetic.
 __device__ __forceinline__ void dma16(uint32_t lane_offset, const void* uniform_base, uint32_t lds_addr) {
