@@ -54,7 +54,9 @@ constexpr int kXcds = 8;
 constexpr int kDmaHalf = kSlotBytes / (kThreads * 16);  // 4 copies per thread and operand slot
 constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, second half B rows
 
-template <int MODE>
+// STREAM: the weight rows are copied with the non-temporal hint.  Right when most experts fit one row tile
+// (every weight byte is then read by one workgroup only); wrong when several row tiles share them through L2.
+template <int MODE, bool STREAM>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
                                                                int ntiles_n, int kslice) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -158,8 +160,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
               dma_base + (stage_k & 1) * kSlotBytes + n * 8192);
     };
     auto copy_b = [&](int n, int stage_k, int slot) {
-        dma16(voff[kDmaHalf + n], base_b + static_cast<int64_t>(stage_k) * (kTK * 2),
-              dma_base + kOffB + slot * kSlotBytes + n * 8192);
+        if (STREAM)
+            dma16_stream(voff[kDmaHalf + n], base_b + static_cast<int64_t>(stage_k) * (kTK * 2),
+                         dma_base + kOffB + slot * kSlotBytes + n * 8192);
+        else
+            dma16(voff[kDmaHalf + n], base_b + static_cast<int64_t>(stage_k) * (kTK * 2),
+                  dma_base + kOffB + slot * kSlotBytes + n * 8192);
     };
     auto issue_a = [&](int stage_k) {
 #pragma unroll
@@ -409,19 +415,32 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev]) {
-        hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_kernel<1>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_kernel<2>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e1 != hipSuccess) return static_cast<int>(e1);
-        if (e2 != hipSuccess) return static_cast<int>(e2);
+        const void* kernels[4] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<1, true>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true>)};
+        for (const void* k : kernels) {
+            hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return static_cast<int>(e);
+        }
         attr_set[dev] = true;
     }
-    if (mode == 1)
-        hipLaunchKernelGGL(gemm_tile_kernel<1>, dim3(grid, 1), dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, p.H);
-    else
-        hipLaunchKernelGGL(gemm_tile_kernel<2>, dim3(grid, static_cast<unsigned>(p.ksplit)), dim3(kThreads), lds_bytes,
-                           s, p, seg_begin, ntiles_n, p.I / p.ksplit);
+    // one row tile per expert on average up to 7/8 full: weights are read once -> streaming copies
+    const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * 7;
+    const dim3 grid1(grid, 1), grid2(grid, static_cast<unsigned>(p.ksplit));
+    if (mode == 1) {
+        if (stream_b)
+            hipLaunchKernelGGL((gemm_tile_kernel<1, true>), grid1, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, p.H);
+        else
+            hipLaunchKernelGGL((gemm_tile_kernel<1, false>), grid1, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, p.H);
+    } else {
+        if (stream_b)
+            hipLaunchKernelGGL((gemm_tile_kernel<2, true>), grid2, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n,
+                               p.I / p.ksplit);
+        else
+            hipLaunchKernelGGL((gemm_tile_kernel<2, false>), grid2, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n,
+                               p.I / p.ksplit);
+    }
     return launch_status();
 }
 

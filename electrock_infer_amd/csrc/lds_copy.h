@@ -29,6 +29,10 @@ __device__ __forceinline__ void dma16(uint32_t lane_offset, const void* uniform_
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(lane_offset), "s"(uniform_base), "s"(lds_addr) : "memory", "m0");
 }
+__device__ __forceinline__ void dma16_stream(uint32_t lane_offset, const void* uniform_base, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                 :: "v"(lane_offset), "s"(uniform_base), "s"(lds_addr) : "memory", "m0");
+}
 template <int N>
 __device__ __forceinline__ void wait_dma() {  // at most N of this wave's copies still in flight
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
