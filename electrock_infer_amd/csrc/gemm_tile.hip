@@ -50,6 +50,7 @@ constexpr int kOffB = kSlotsA * kSlotBytes;          // B ring behind the A ring
 constexpr int kLdsBytes = (kSlotsA + kSlotsB) * kSlotBytes;  // 160 KB
 constexpr int kRowBlock = 32;                        // sort padding this kernel needs
 constexpr int kGroupM = 4;
+constexpr int kMaxGroupRows = 12;                  // row tiles of one expert that share a pass over its weights
 constexpr int kXcds = 8;
 constexpr int kDmaHalf = kSlotBytes / (kThreads * 16);  // 4 copies per thread and operand slot
 constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, second half B rows
@@ -80,8 +81,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             local -= t;
         }
         const int rows_e = (seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM;
-        nt = xcd * cols + local / rows_e;
-        mt = local % rows_e;
+        // experts with many row tiles are walked in groups of at most kMaxGroupRows row tiles (else the CUs of
+        // an XCD would share one weight tile but no token rows)
+        const int ngroups = (rows_e + kMaxGroupRows - 1) / kMaxGroupRows;
+        const int grows = (rows_e + ngroups - 1) / ngroups;
+        int g0 = 0, gr = grows;
+        for (;; g0 += grows) {
+            gr = (rows_e - g0 < grows) ? rows_e - g0 : grows;
+            if (local < gr * cols) break;
+            local -= gr * cols;
+        }
+        nt = xcd * cols + local / gr;
+        mt = g0 + local % gr;
     } else {
         // column count not divisible: contiguous ranges of 4 row tiles x all column tiles per XCD
         const int total = mtiles * ntiles_n;
