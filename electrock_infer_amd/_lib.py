@@ -15,6 +15,7 @@ ITYPE_I32, ITYPE_I64 = 0, 1
 
 FLAG_OUT_F32 = 1 << 0
 FLAG_ACCURATE = 1 << 1
+FLAG_GATE_F32_LOGITS = 1 << 2
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10
@@ -26,7 +27,7 @@ FLAG_FORCE_GENERIC = 1 << 16
 EXPORTED_SYMBOLS = (
     "em_version", "em_error_string", "em_topk_softmax", "em_moe_align_block_size",
     "em_silu_and_mul", "em_moe_sum", "em_moe_workspace_bytes", "em_moe_workspace_layout",
-    "em_moe_forward",
+    "em_moe_forward", "em_moe_forward_gated", "em_gate_topk_softmax",
 )
 
 
@@ -70,6 +71,10 @@ def load() -> ctypes.CDLL:
     lib.em_moe_workspace_layout.argtypes = [i64, i32, i32, i32, i32, ctypes.POINTER(MoeLayout)]
     lib.em_moe_forward.restype = i32
     lib.em_moe_forward.argtypes = [vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
+    lib.em_moe_forward_gated.restype = i32
+    lib.em_moe_forward_gated.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
+    lib.em_gate_topk_softmax.restype = i32
+    lib.em_gate_topk_softmax.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp]
     _lib = lib
     return lib
 

@@ -148,13 +148,21 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k) {
     return static_cast<size_t>(L.total_bytes);
 }
 
-int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, const void* w13,
-                   const void* w2, void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
-                   void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// The layer behind both entry points: the routing comes either from caller-provided logits or from the
+// gate matrix (gate_w != nullptr: logits = x . gate_w^T computed in the router's launch).
+int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype, const void* gate_w, const void* w13,
+                     const void* w2, void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
+                     void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
     if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
-    if (!dtype_ok(logits_dtype)) return EM_ERR_BAD_DTYPE;
+    if (gate_w == nullptr && !dtype_ok(logits_dtype)) return EM_ERR_BAD_DTYPE;
+    if (gate_w != nullptr && !gate_router_supported(H, E)) return EM_ERR_UNSUPPORTED;
     if (T == 0) return 0;
-    if (!x || !router_logits || !w13 || !w2 || !out || !workspace) return EM_ERR_NULL_POINTER;
+    if (!x || (!router_logits && !gate_w) || !w13 || !w2 || !out || !workspace) return EM_ERR_NULL_POINTER;
+    if (gate_w != nullptr && !aligned(gate_w, 16)) return EM_ERR_ALIGNMENT;
     if (!aligned(x, 16) || !aligned(w13, 16) || !aligned(w2, 16) || !aligned(out, 16) ||
         !aligned(workspace, 256))
         return EM_ERR_ALIGNMENT;
@@ -194,7 +202,10 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
     p.ksplit = static_cast<int>(L.ksplit);
 
     if (!(flags & EM_FLAG_SKIP_ROUTER)) {
-        rc = launch_router(router_logits, logits_dtype, T, E, top_k, renormalize, topk_w, topk_ids, s);
+        rc = gate_w != nullptr
+                 ? launch_gate_router(x, gate_w, T, H, E, top_k, renormalize, (flags & EM_FLAG_GATE_F32_LOGITS) ? 0 : 1,
+                                      nullptr, topk_w, topk_ids, s)
+                 : launch_router(router_logits, logits_dtype, T, E, top_k, renormalize, topk_w, topk_ids, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_ALIGN)) {
@@ -234,6 +245,37 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
         if (rc != 0) return rc;
     }
     return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, const void* w13,
+                   const void* w2, void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
+                   void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    return moe_forward_impl(x, router_logits, logits_dtype, nullptr, w13, w2, out, T, H, I, E, top_k, renormalize,
+                            workspace, workspace_bytes, flags, stream);
+}
+
+int em_moe_forward_gated(const void* x, const void* gate_w, const void* w13, const void* w2, void* out,
+                         int64_t T, int H, int I, int E, int top_k, int renormalize, void* workspace,
+                         size_t workspace_bytes, unsigned flags, void* stream) {
+    if (!gate_w && T > 0 && shapes_ok(T, H, I, E, top_k)) return EM_ERR_NULL_POINTER;
+    return moe_forward_impl(x, nullptr, EM_DTYPE_BF16, gate_w, w13, w2, out, T, H, I, E, top_k, renormalize, workspace,
+                            workspace_bytes, flags, stream);
+}
+
+int em_gate_topk_softmax(const void* x, const void* gate_w, int64_t T, int H, int E, int k, int renormalize,
+                         int round_logits_bf16, void* logits_out, float* topk_weights, int32_t* topk_ids,
+                         void* stream) {
+    if (T < 0 || H <= 0 || H % 8 != 0 || E < 1 || E > kMaxExperts || k < 1 || k > E) return EM_ERR_BAD_SHAPE;
+    if (!gate_router_supported(H, E)) return EM_ERR_UNSUPPORTED;
+    if (T == 0) return 0;
+    if (!x || !gate_w || !topk_weights || !topk_ids) return EM_ERR_NULL_POINTER;
+    if (!aligned(x, 16) || !aligned(gate_w, 16)) return EM_ERR_ALIGNMENT;
+    return launch_gate_router(x, gate_w, T, H, E, k, renormalize, round_logits_bf16 ? 1 : 0, logits_out, topk_weights,
+                              topk_ids, as_stream(stream));
 }
 
 }  // extern "C"

@@ -81,6 +81,9 @@ inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 // ---- stage launchers (defined in the .hip files, called from capi.hip) ------
 int launch_router(const void* logits, int logits_dtype, int64_t T, int E, int k, int renorm,
                   float* w, int32_t* ids, hipStream_t s);
+bool gate_router_supported(int H, int E);
+int launch_gate_router(const void* x, const void* gate_w, int64_t T, int H, int E, int k, int renorm,
+                       int round_bf16, void* logits_out, float* w, int32_t* ids, hipStream_t s);
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
                  int32_t* post_pad, int32_t* seg_out /* [E+1] padded segment starts, may be null */,

@@ -6,7 +6,7 @@
 // (selection on raw logits, strict '>' in ascending expert order, hence ties go
 // to the lowest index; weight = exp(x - max) / sum) and, when renorm is set,
 // fused_moe.py:161-162 (weights divided by the sum of the selected ones).
-#include "common.h"
+#include "router_device.h"
 
 namespace em {
 namespace {
@@ -26,45 +26,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_kernel(
         v = Elem::load(logits[t * E + lane]);
         if (v != v) v = -INFINITY;  // a NaN logit can never be selected
     }
-
-    // row max and softmax denominator
-    float mx = v;
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    const float ex = (lane < E) ? expf(v - mx) : 0.0f;
-    float denom = ex;
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) denom += __shfl_xor(denom, off);
-
-    // k rounds of arg-max over the lanes still alive.  (alive desc, value desc,
-    // index asc) is a total order, so every lane ends a round with the same
-    // winner; retired lanes and lanes >= E can never win while k <= E, which
-    // keeps the k indices distinct and in [0, E) even for rows of -inf.
-    int alive = (lane < E) ? 1 : 0;
-    float my_w = 0.0f;  // lane j < k keeps the j-th selected weight
-    int my_id = 0;
-    float sel_sum = 0.0f;
-    for (int j = 0; j < k; ++j) {
-        int ba = alive;
-        float bv = v;
-        int bi = lane;
-#pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) {
-            const int oa = __shfl_xor(ba, off);
-            const float ov = __shfl_xor(bv, off);
-            const int oi = __shfl_xor(bi, off);
-            const bool better = (oa > ba) || (oa == ba && (ov > bv || (ov == bv && oi < bi)));
-            if (better) { ba = oa; bv = ov; bi = oi; }
-        }
-        const float p = __shfl(ex, bi) / denom;
-        sel_sum += p;
-        if (lane == j) { my_w = p; my_id = bi; }
-        if (lane == bi) alive = 0;
-    }
-    if (lane < k) {
-        out_w[t * k + lane] = renorm ? my_w / sel_sum : my_w;
-        out_ids[t * k + lane] = my_id;
-    }
+    route_from_logit(v, lane, t, E, k, renorm, out_w, out_ids);
 }
 
 }  // namespace

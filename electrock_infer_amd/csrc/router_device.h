@@ -1,0 +1,54 @@
+// Router selection shared by the stand-alone router and by the kernel that computes the logits itself.
+#pragma once
+#include "common.h"
+
+namespace em {
+
+// One token, executed by one whole wavefront: lane e < E brings the logit of expert e in `v`
+// (a NaN logit must already be -inf), the k selected weights and ids go to out_w / out_ids [t*k .. t*k+k).
+// Selection on the raw logits, strict '>' in ascending expert order, hence ties go to the lowest index
+// (src/topk_softmax_kernels.hip:23-64); weight = exp(x - max) / sum, divided by the sum of the selected
+// ones when renorm is set (fused_moe.py:161-162).
+__device__ __forceinline__ void route_from_logit(float v, int lane, int64_t t, int E, int k, int renorm,
+                                                 float* __restrict__ out_w, int32_t* __restrict__ out_ids) {
+    // row max and softmax denominator
+    float mx = v;
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    const float ex = (lane < E) ? expf(v - mx) : 0.0f;
+    float denom = ex;
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) denom += __shfl_xor(denom, off);
+
+    // k rounds of arg-max over the lanes still alive.  (alive desc, value desc,
+    // index asc) is a total order, so every lane ends a round with the same
+    // winner; retired lanes and lanes >= E can never win while k <= E, which
+    // keeps the k indices distinct and in [0, E) even for rows of -inf.
+    int alive = (lane < E) ? 1 : 0;
+    float my_w = 0.0f;  // lane j < k keeps the j-th selected weight
+    int my_id = 0;
+    float sel_sum = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        int ba = alive;
+        float bv = v;
+        int bi = lane;
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const int oa = __shfl_xor(ba, off);
+            const float ov = __shfl_xor(bv, off);
+            const int oi = __shfl_xor(bi, off);
+            const bool better = (oa > ba) || (oa == ba && (ov > bv || (ov == bv && oi < bi)));
+            if (better) { ba = oa; bv = ov; bi = oi; }
+        }
+        const float p = __shfl(ex, bi) / denom;
+        sel_sum += p;
+        if (lane == j) { my_w = p; my_id = bi; }
+        if (lane == bi) alive = 0;
+    }
+    if (lane < k) {
+        out_w[t * k + lane] = renorm ? my_w / sel_sum : my_w;
+        out_ids[t * k + lane] = my_id;
+    }
+}
+
+}  // namespace em

@@ -141,3 +141,70 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         _lib.current_stream(hidden_states.device))
     _lib.check(code, "fused_experts")
     return output
+
+
+def gate_topk(hidden_states: torch.Tensor, gate_weight: torch.Tensor, topk: int, renormalize: bool = True,
+              bf16_logits: bool = True, return_logits: bool = False):
+    """Router gate and router in one launch: ``fused_topk(hidden_states, F.linear(hidden_states, gate_weight), ...)``
+    (models/mixtral.py:59 followed by fused_moe.py:130-164).
+
+    hidden_states [T, H] bf16, gate_weight [E, H] bf16 (``nn.Linear`` layout).  With ``bf16_logits`` the fp32 dot
+    products are rounded to bf16 before the selection, as the reference's bf16 linear layer returns them.
+    Returns (topk_weights [T, topk] fp32, topk_ids [T, topk] int32[, logits [T, E]]).
+    """
+    _lib.require_device(hidden_states, gate_weight)
+    T, H = hidden_states.shape
+    E = gate_weight.shape[0]
+    if gate_weight.shape[1] != H:
+        raise RuntimeError("gate_weight must be [num_experts, hidden_size]")
+    if not (hidden_states.dtype == gate_weight.dtype == torch.bfloat16):
+        raise RuntimeError("the router gate computes in bfloat16: hidden_states and gate_weight must be bfloat16")
+    dev = hidden_states.device
+    topk_weights = torch.empty(T, topk, dtype=torch.float32, device=dev)
+    topk_ids = torch.empty(T, topk, dtype=torch.int32, device=dev)
+    logits = torch.empty(T, E, dtype=torch.bfloat16 if bf16_logits else torch.float32, device=dev) if return_logits else None
+    code = _lib.load().em_gate_topk_softmax(
+        hidden_states.data_ptr(), gate_weight.data_ptr(), T, H, E, topk, 1 if renormalize else 0,
+        1 if bf16_logits else 0, logits.data_ptr() if logits is not None else None,
+        topk_weights.data_ptr(), topk_ids.data_ptr(), _lib.current_stream(dev))
+    _lib.check(code, "gate_topk")
+    return (topk_weights, topk_ids, logits) if return_logits else (topk_weights, topk_ids)
+
+
+def fused_experts_gated(hidden_states: torch.Tensor, gate_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                        topk: int, renormalize: bool = True, inplace: bool = False,
+                        out_dtype: Optional[torch.dtype] = None, accurate: bool = False, bf16_logits: bool = True,
+                        flags: int = 0, workspace: Optional[MoeWorkspace] = None) -> torch.Tensor:
+    """``fused_experts(x, w1, w2, F.linear(x, gate_weight), ...)`` in one call: the whole MoE block of the model
+    (models/mixtral.py:53-63) with the router gate computed inside the router's launch."""
+    _lib.require_device(hidden_states, gate_weight, w1, w2)
+    T, H = hidden_states.shape
+    E, two_i, Hw = w1.shape
+    I = two_i // 2
+    if Hw != H or tuple(w2.shape) != (E, H, I) or two_i != 2 * I:
+        raise RuntimeError("weight shapes do not match hidden_states")
+    if tuple(gate_weight.shape) != (E, H):
+        raise RuntimeError("gate_weight must be [num_experts, hidden_size]")
+    if not (hidden_states.dtype == gate_weight.dtype == w1.dtype == w2.dtype == torch.bfloat16):
+        raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, gate_weight, w1 and w2 must be bfloat16")
+    want_f32 = out_dtype == torch.float32
+    if accurate:
+        flags |= _lib.FLAG_ACCURATE
+    if not bf16_logits:
+        flags |= _lib.FLAG_GATE_F32_LOGITS
+    if want_f32 and inplace:
+        raise RuntimeError("a float32 result cannot be written in place over bfloat16 hidden_states")
+    if want_f32:
+        output = torch.empty((T, H), dtype=torch.float32, device=hidden_states.device)
+        flags |= _lib.FLAG_OUT_F32
+    else:
+        output = hidden_states if inplace else torch.empty_like(hidden_states)
+    if T == 0:
+        return output
+    ws = workspace or get_workspace(hidden_states.device, T, H, I, E, topk)
+    code = _lib.load().em_moe_forward_gated(
+        hidden_states.data_ptr(), gate_weight.data_ptr(), w1.data_ptr(), w2.data_ptr(), output.data_ptr(),
+        T, H, I, E, topk, 1 if renormalize else 0, ws.buffer.data_ptr(), ctypes.c_size_t(ws.buffer.numel()), flags,
+        _lib.current_stream(hidden_states.device))
+    _lib.check(code, "fused_experts_gated")
+    return output

@@ -45,6 +45,8 @@ extern "C" {
 /* em_moe_forward flags */
 #define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16      */
 #define EM_FLAG_ACCURATE       (1u << 1)  /* SiLU*mul activations kept as a bf16 hi+lo pair  */
+#define EM_FLAG_GATE_F32_LOGITS (1u << 2) /* em_moe_forward_gated: route on the fp32 logits,   */
+                                          /* not on their bf16 rounding                        */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
 #define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
 #define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
@@ -74,6 +76,26 @@ const char* em_error_string(int code);
 int em_topk_softmax(const void* logits, int logits_dtype, int64_t T, int E, int k,
                     int renormalize, float* topk_weights, int32_t* topk_ids,
                     void* stream);
+
+/*
+ * Router gate and router in one launch: logits = x . gate_w^T, then em_topk_softmax.
+ * Replaces the gate of the model's MoE block plus the router call behind it:
+ *   router_logits = self.gate(hidden_states)        (models/mixtral.py:40-42,59;
+ *   ReplicatedLinear = F.linear(x, weight), layers/linear.py:31-54), followed by
+ *   fused_topk (layers/moe/fused_moe.py:130-164).
+ * The dot products are accumulated in fp32.  With round_logits_bf16 != 0 each logit is then
+ * rounded to bf16, as the reference's bf16 linear layer returns it (equal logits exist in
+ * that case and go to the lowest expert index); with 0 the fp32 sums are used directly.
+ *   x             [T, H]  bf16, 16-byte aligned
+ *   gate_w        [E, H]  bf16, 16-byte aligned (nn.Linear weight layout)
+ *   logits_out    [T, E]  optional (may be NULL): the logits that were routed on, bf16 when
+ *                         round_logits_bf16 != 0, float32 otherwise
+ *   topk_weights  [T, k]  float32, topk_ids [T, k] int32, as em_topk_softmax
+ * Limits: E in {8, 16}, H % 8 == 0, E * H * 2 <= 160 KiB (the gate matrix is kept in LDS).
+ */
+int em_gate_topk_softmax(const void* x, const void* gate_w, int64_t T, int H, int E, int k,
+                         int renormalize, int round_logits_bf16, void* logits_out,
+                         float* topk_weights, int32_t* topk_ids, void* stream);
 
 /*
  * Expert sort with padding to the GEMM block size.
@@ -154,6 +176,16 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype,
                    int64_t T, int H, int I, int E, int top_k, int renormalize,
                    void* workspace, size_t workspace_bytes, unsigned flags,
                    void* stream);
+
+/*
+ * The same layer with the router gate inside: replaces MixtralMoE.forward
+ * (models/mixtral.py:53-63: gate -> experts) in one call.  Arguments as em_moe_forward, with
+ * gate_w [E, H] bf16 in place of router_logits; EM_FLAG_GATE_F32_LOGITS routes on the fp32
+ * logits instead of their bf16 rounding.  Limits of em_gate_topk_softmax apply.
+ */
+int em_moe_forward_gated(const void* x, const void* gate_w, const void* w13, const void* w2,
+                         void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
+                         void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
 
 /*
  * Byte offsets and element counts of the routing results em_moe_forward leaves

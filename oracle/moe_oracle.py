@@ -43,6 +43,30 @@ def get_moe_config(num_tokens: int, num_experts: int) -> dict:
 
 
 # ----------------------------------------------------------------------------
+# A9  router gate (the caller's step in front of the layer)
+# ----------------------------------------------------------------------------
+def to_bf16_f32(a: np.ndarray) -> np.ndarray:
+    """Round float32 to the nearest bfloat16 (ties to even), returned as float32."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def gate_logits(x: np.ndarray, gate_w: np.ndarray, round_bf16: bool = True) -> np.ndarray:
+    """Router logits of the model's MoE block: ``F.linear(x, weight)`` without bias
+    (models/mixtral.py:40-42,59; layers/linear.py:53-54).
+
+    x [T, H], gate_w [E, H] (values of bf16 tensors, any float dtype).  The dot products are
+    taken in float64 and rounded once to float32 (a bf16 linear layer accumulates in fp32;
+    its summation order is the library's), then to bf16 when ``round_bf16`` -- what the
+    reference's bf16 linear returns.  -> float32 [T, E].
+    """
+    acc = np.asarray(x, dtype=np.float64) @ np.asarray(gate_w, dtype=np.float64).T
+    out = acc.astype(np.float32)
+    return to_bf16_f32(out) if round_bf16 else out
+
+
+# ----------------------------------------------------------------------------
 # A1/A2  router
 # ----------------------------------------------------------------------------
 def topk_softmax(logits: np.ndarray, topk: int, renormalize: bool) -> Tuple[np.ndarray, np.ndarray]:

@@ -80,6 +80,33 @@ def test_router_invariants_with_bf16_ties():
 
 
 # ----------------------------------------------------------------- align ----
+def test_gate_logits_hand_worked_and_library():
+    # hand-worked: two tokens, two experts, exact small integers
+    x = np.array([[1.0, 2.0, -3.0, 0.5], [0.0, -1.0, 4.0, 2.0]], dtype=np.float32)
+    w = np.array([[2.0, 0.0, 1.0, 4.0], [-1.0, 1.0, 0.5, -2.0]], dtype=np.float32)
+    #   token 0: [2 + 0 - 3 + 2, -1 + 2 - 1.5 - 1] = [1, -1.5];  token 1: [0 + 0 + 4 + 8, 0 - 1 + 2 - 4] = [12, -3]
+    np.testing.assert_array_equal(O.gate_logits(x, w, round_bf16=False), np.array([[1.0, -1.5], [12.0, -3.0]], np.float32))
+    # library routine: float64 linear layer of torch, rounded once; and torch's own bf16 rounding of the result
+    g = torch.Generator().manual_seed(3)
+    xt = torch.randn(37, 256, generator=g).to(torch.bfloat16)
+    wt = (torch.randn(8, 256, generator=g) * 0.05).to(torch.bfloat16)
+    ref64 = torch.nn.functional.linear(xt.double(), wt.double())
+    got = O.gate_logits(xt.float().numpy(), wt.float().numpy(), round_bf16=False)
+    np.testing.assert_array_equal(got, ref64.float().numpy())
+    got_bf = O.gate_logits(xt.float().numpy(), wt.float().numpy(), round_bf16=True)
+    np.testing.assert_array_equal(got_bf, ref64.float().to(torch.bfloat16).float().numpy())
+    # a transposed weight or a dropped element changes the result
+    assert not np.array_equal(O.gate_logits(x, w[::-1], round_bf16=False), O.gate_logits(x, w, round_bf16=False))
+
+
+def test_to_bf16_rounding_is_nearest_even():
+    # 1 + 2^-8 is exactly between bf16 1.0 and 1.0078125 -> even mantissa (1.0); 1 + 3 * 2^-8 -> 1.015625
+    a = np.array([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, -(1.0 + 2.0 ** -8), 3.0e38, 1e-40], dtype=np.float32)
+    want = torch.from_numpy(a).to(torch.bfloat16).float().numpy()
+    np.testing.assert_array_equal(O.to_bf16_f32(a), want)
+    assert O.to_bf16_f32(a)[0] == 1.0 and O.to_bf16_f32(a)[1] == 1.015625
+
+
 def test_align_hand_worked():
     # slots 0..5 -> experts [2,0,2,1,0,2], E=3, block 2:
     # counts 2,1,3 -> padded 2,2,4 -> offsets 0,2,4, total 8
