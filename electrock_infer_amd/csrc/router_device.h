@@ -4,51 +4,61 @@
 
 namespace em {
 
-// One token, executed by one whole wavefront: lane e < E brings the logit of expert e in `v`
-// (a NaN logit must already be -inf), the k selected weights and ids go to out_w / out_ids [t*k .. t*k+k).
+// One token per aligned group of G lanes (G a power of two, E <= G <= 64): lane `sub` < E of the group brings
+// the logit of expert `sub` in `v` (a NaN logit must already be -inf), the k selected weights and ids go to
+// out_w / out_ids [t*k .. t*k+k) when `valid`.  All 64 lanes of the wavefront must call it together.
 // Selection on the raw logits, strict '>' in ascending expert order, hence ties go to the lowest index
 // (src/topk_softmax_kernels.hip:23-64); weight = exp(x - max) / sum, divided by the sum of the selected
 // ones when renorm is set (fused_moe.py:161-162).
-__device__ __forceinline__ void route_from_logit(float v, int lane, int64_t t, int E, int k, int renorm,
-                                                 float* __restrict__ out_w, int32_t* __restrict__ out_ids) {
+template <int G>
+__device__ __forceinline__ void route_group(float v, int lane, int64_t t, bool valid, int E, int k, int renorm,
+                                            float* __restrict__ out_w, int32_t* __restrict__ out_ids) {
+    const int sub = lane & (G - 1);
+    const int group_base = lane - sub;
     // row max and softmax denominator
     float mx = v;
 #pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    const float ex = (lane < E) ? expf(v - mx) : 0.0f;
+    for (int off = G / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    const float ex = (sub < E) ? expf(v - mx) : 0.0f;
     float denom = ex;
 #pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) denom += __shfl_xor(denom, off);
+    for (int off = G / 2; off > 0; off >>= 1) denom += __shfl_xor(denom, off);
 
     // k rounds of arg-max over the lanes still alive.  (alive desc, value desc,
-    // index asc) is a total order, so every lane ends a round with the same
+    // index asc) is a total order, so every lane of a group ends a round with the same
     // winner; retired lanes and lanes >= E can never win while k <= E, which
     // keeps the k indices distinct and in [0, E) even for rows of -inf.
-    int alive = (lane < E) ? 1 : 0;
+    int alive = (sub < E) ? 1 : 0;
     float my_w = 0.0f;  // lane j < k keeps the j-th selected weight
     int my_id = 0;
     float sel_sum = 0.0f;
     for (int j = 0; j < k; ++j) {
         int ba = alive;
         float bv = v;
-        int bi = lane;
+        int bi = sub;
 #pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) {
+        for (int off = G / 2; off > 0; off >>= 1) {
             const int oa = __shfl_xor(ba, off);
             const float ov = __shfl_xor(bv, off);
             const int oi = __shfl_xor(bi, off);
             const bool better = (oa > ba) || (oa == ba && (ov > bv || (ov == bv && oi < bi)));
             if (better) { ba = oa; bv = ov; bi = oi; }
         }
-        const float p = __shfl(ex, bi) / denom;
+        const float p = __shfl(ex, group_base + bi) / denom;
         sel_sum += p;
-        if (lane == j) { my_w = p; my_id = bi; }
-        if (lane == bi) alive = 0;
+        if (sub == j) { my_w = p; my_id = bi; }
+        if (sub == bi) alive = 0;
     }
-    if (lane < k) {
-        out_w[t * k + lane] = renorm ? my_w / sel_sum : my_w;
-        out_ids[t * k + lane] = my_id;
+    if (valid && sub < k) {
+        out_w[t * k + sub] = renorm ? my_w / sel_sum : my_w;
+        out_ids[t * k + sub] = my_id;
     }
+}
+
+// One token per wavefront: lane e < E brings the logit of expert e.
+__device__ __forceinline__ void route_from_logit(float v, int lane, int64_t t, int E, int k, int renorm,
+                                                 float* __restrict__ out_w, int32_t* __restrict__ out_ids) {
+    route_group<kWave>(v, lane, t, true, E, k, renorm, out_w, out_ids);
 }
 
 }  // namespace em

@@ -37,9 +37,12 @@ def test_gate_topk_matches_oracle(T, H, E, bf16_logits):
     if bf16_logits:
         # the fp32 sums differ from the oracle's in the last bits (summation order), so a logit that sits on a
         # rounding boundary may land on the neighbouring bf16 value: at most one bf16 step, and rarely
-        step = np.abs(got - want) / bf16_ulp(want)
-        assert step.max() <= 1.0 + 1e-6
-        assert (step > 0).mean() < 2e-3
+        # (for logits near zero a bf16 step is smaller than the fp32 rounding of the partial sums, whose size
+        # follows sum |x_i * g_i|: allow that on top)
+        sum_abs = np.abs(x.float().cpu().numpy()).astype(np.float64) @ np.abs(gw.float().cpu().numpy()).astype(np.float64).T
+        err = np.abs(got - want)
+        assert (err <= bf16_ulp(want) * (1.0 + 1e-6) + 4 * 2.0 ** -24 * sum_abs).all()
+        assert (err > 0).mean() < 2e-3
     else:
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
     # the selection must be the oracle's selection on the logits the kernel itself produced (bit-exact ids),
