@@ -23,12 +23,16 @@
 //              a SIMD at once) they left the matrix pipe idle for a fifth of every step
 //   LDS        rows are 128 B; the 16-byte pieces of every 2-row group are XOR-
 //              swizzled so that the 16 lanes of a b128 operand read hit 16 bank groups
-//   wave       128 x 64 sub-tile = 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (the
-//              16x16x32 form runs at half this rate on gfx950); operand fragments are
+//   wave       128 x 64 sub-tile = 8 x 4 v_mfma_f32_16x16x32_bf16 accumulators.  Both bf16
+//              shapes run at the same rate, but with real operand values the board's power
+//              limit, not the issue rate, sets the speed, and this shape needs less power
+//              per flop (registers-only loop, N(0,1) x N(0,0.02) operands: 2.08 against
+//              1.85 PFLOP/s for 32x32x16).  A K step of 64 is walked in four units of 16
+//              MFMAs (upper / lower 64 rows x first / second 32 of K); operand fragments are
 //              double-buffered in registers and their LDS reads are woven between the
-//              MFMAs of the previous 16-wide K step, also across the stage barrier
-//   MODE 1     the wave's two N fragments are 32 gate rows j and the matching 32
-//              up rows I + j, so SiLU(g) * u is lane-local in the epilogue
+//              MFMAs of the previous unit, also across the stage barrier
+//   MODE 1     N fragments 0, 1 of a wave are 32 gate rows j and fragments 2, 3 the matching
+//              32 up rows I + j, so SiLU(g) * u is lane-local in the epilogue
 //   MODE 2     256 rows of w2[e], optionally one of `ksplit` K slices; fp32 partial rows
 //              are scattered to y[z, slot]
 //   order      workgroup ids are dealt to the 8 XCDs round-robin by the hardware; each XCD
@@ -188,61 +192,73 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         for (int n = 0; n < kDmaHalf; ++n) copy_b(n, stage_k, slot);
     };
 
-    f32x16_t acc[4][2];
+    // accumulator (f, g): rows wm*128 + f*16 .. +16 of the tile, weight rows wn*64 + g*16 .. +16
+    f32x4_t acc[8][4];
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+    for (int f = 0; f < 8; ++f)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
+        for (int g = 0; g < 4; ++g) acc[f][g] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // ---- operand reads: lane (r32, kh) takes row r32 of a 32-row fragment, piece ks*2 + kh ----
-    const int r32 = lane & 31;
-    const int kh = lane >> 5;
-    const int sw = (r32 >> 1) & 7;  // (row / 2) & 7 is the same for every fragment of this lane
-    int a_off[4], b_off[4];
+    // ---- operand reads: lane (r16, kq) takes row r16 of a 16-row fragment, piece k32*4 + kq of the 128-byte row ----
+    const int r16 = lane & 15;
+    const int kq = lane >> 4;
+    const int sw = (r16 >> 1) & 7;  // (row / 2) & 7 is the same for every fragment of this lane
+    int a_off[2], b_off[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        const int piece = (ks * 2 + kh) ^ sw;
-        const int ra = wm * 128 + r32, rb = wn * 64 + r32;
-        a_off[ks] = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
-        b_off[ks] = kOffB + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
+    for (int k32 = 0; k32 < 2; ++k32) {
+        const int piece = (k32 * 4 + kq) ^ sw;
+        const int ra = wm * 128 + r16, rb = wn * 64 + r16;
+        a_off[k32] = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
+        b_off[k32] = kOffB + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
     }
-    // 32-row fragments of this wave that hold rows of the tile (wave-uniform)
+    // 32-row blocks of this wave that hold rows of the tile (wave-uniform); 16-row fragment f exists if f < 2 * nmi
     int nmi = (valid - wm * 128 + 31) / 32;
     nmi = nmi < 0 ? 0 : (nmi > 4 ? 4 : nmi);
     nmi = __builtin_amdgcn_readfirstlane(nmi);
 
-    bf16x8_t fa[2][4], fb[2][2];
-    // operand fragments of 16-wide K step ks of K step stage_k (weight rows in ring slot bslot) -> register set `set`
-    auto read_frags = [&](int stage_k, int bslot, int ks, int set, auto full_tag) {
+    // Unit u = 0..3 of a K step: row half h = u & 1 (fragments 4h .. 4h+3), K half k32 = u >> 1.
+    // Token fragments live in register set u & 1, weight fragments (shared by both row halves) in set k32.
+    bf16x8_t fa[2][4], fb[2][4];
+    // operand fragments of unit u of K step stage_k (weight rows in ring slot bslot)
+    auto read_frags = [&](int stage_k, int bslot, int u, auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;
+        const int h = u & 1, k32 = u >> 1;
         const uint8_t* sa = smem + (stage_k & 1) * kSlotBytes;
         const uint8_t* sb = smem + bslot * kSlotBytes;
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
-            if (FULL || mi < nmi) fa[set][mi] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[ks] + mi * 4096);
+        for (int j = 0; j < 4; ++j)
+            if (FULL || h * 4 + j < 2 * nmi)
+                fa[h][j] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[k32] + (h * 4 + j) * 2048);
+        if (h == 0) {
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[ks] + ni * 4096);
-    };
-    auto multiply = [&](int set, auto full_tag) {
-        constexpr bool FULL = decltype(full_tag)::value;
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
-            if (FULL || mi < nmi) {
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
-            }
-        if (FULL) {  // scheduling hint: one LDS read after each of the first six MFMAs, then the last two
-#pragma unroll
-            for (int i = 0; i < 6; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            for (int g = 0; g < 4; ++g) fb[k32][g] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[k32] + g * 2048);
         }
     };
+    // the 16 MFMAs of unit u; `reads` LDS reads issued just before the call are spread one behind each of the first MFMAs
+    auto multiply = [&](int u, auto reads_tag, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        constexpr int reads = decltype(reads_tag)::value;
+        const int h = u & 1, k32 = u >> 1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (FULL || h * 4 + j < 2 * nmi) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    acc[h * 4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[h][j], fb[k32][g], acc[h * 4 + j][g], 0, 0, 0);
+            }
+        if (FULL) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i < reads) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            __builtin_amdgcn_sched_group_barrier(0x008, 16 - reads, 0);
+        }
+    };
+    const std::integral_constant<int, 0> r0;
+    const std::integral_constant<int, 4> r4;
+    const std::integral_constant<int, 8> r8;
     auto next_slot = [](int slot) { return slot == kSlotsB - 1 ? 0 : slot + 1; };
 
     // Copies are queued per wave in the order  A(0) B(0) B(1) | A(1) B(2) | A(2) B(3) | ...  so that at the end
@@ -264,12 +280,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         // kt, the eight MFMAs of its last 16-wide K step alternate with the copies of A(kt+2) and B(kt+3) (the
         // slots step kt has just freed) and with the first operand reads of step kt+1.
         const std::true_type full;
-        read_frags(0, 0, 0, 0, full);
+        read_frags(0, 0, 0, full);
         auto step = [&](int kt, auto copy_a_tag, auto copy_b_tag) {
             constexpr bool CA = decltype(copy_a_tag)::value, CB = decltype(copy_b_tag)::value;
-            read_frags(kt, bs, 1, 1, full); multiply(0, full);
-            read_frags(kt, bs, 2, 0, full); multiply(1, full);
-            read_frags(kt, bs, 3, 1, full); multiply(0, full);
+            read_frags(kt, bs, 1, full); multiply(0, r4, full);
+            read_frags(kt, bs, 2, full); multiply(1, r8, full);
+            read_frags(kt, bs, 3, full); multiply(2, r4, full);
             if (CA) wait_dma<kDmaHalf>(); else wait_dma<0>();   // this wave's parts of A(kt+1), B(kt+1) are in LDS
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of step kt are in registers
             block_barrier();                                    // ... and so are everyone else's
@@ -277,12 +293,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             const int bn = next_slot(bs);
             const uint8_t* sa = smem + ((kt + 1) & 1) * kSlotBytes;
             const uint8_t* sb = smem + bn * kSlotBytes;
+            // unit 3 of step kt; behind every second MFMA a copy, behind the others a read of unit 0 of step kt+1
+            // (weight fragment 0 and token fragment 0 first: the next unit starts with them)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i >> 1], fb[1][i & 1], acc[i >> 1][i & 1], 0, 0, 0);
-                if (i < 4) { if (CA) copy_a(i, kt + 2); } else { if (CB) copy_b(i - 4, kt + 3, bs); }
-                if (i < 4) fa[0][i] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0] + i * 4096);
-                else if (i < 6) fb[0][i - 4] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0] + (i - 4) * 4096);
+            for (int i = 0; i < 16; ++i) {
+                acc[4 + (i >> 2)][i & 3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][i >> 2], fb[1][i & 3], acc[4 + (i >> 2)][i & 3], 0, 0, 0);
+                const int n = i >> 1;
+                if ((i & 1) == 0) {
+                    if (n < 4) { if (CA) copy_a(n, kt + 2); } else { if (CB) copy_b(n - 4, kt + 3, bs); }
+                } else if (n == 0) {
+                    fb[0][0] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0]);
+                } else if (n == 1) {
+                    fa[0][0] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0]);
+                } else if (n < 5) {
+                    fb[0][n - 1] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0] + (n - 1) * 2048);
+                } else {
+                    fa[0][n - 4] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0] + (n - 4) * 2048);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             bs = bn;
@@ -291,21 +318,21 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         for (; kt + 3 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
         for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::false_type{});
         for (; kt + 1 < nk; ++kt) step(kt, std::false_type{}, std::false_type{});
-        read_frags(nk - 1, bs, 1, 1, full); multiply(0, full);
-        read_frags(nk - 1, bs, 2, 0, full); multiply(1, full);
-        read_frags(nk - 1, bs, 3, 1, full); multiply(0, full);
-        multiply(1, full);
+        read_frags(nk - 1, bs, 1, full); multiply(0, r4, full);
+        read_frags(nk - 1, bs, 2, full); multiply(1, r8, full);
+        read_frags(nk - 1, bs, 3, full); multiply(2, r4, full);
+        multiply(3, r0, full);
     } else {
         // Short tile: a wave multiplies the fragments that exist; waves without rows still copy and meet the
         // barriers.  Skipped copies of missing token rows do not change the counts: the newest four are B's.
         const std::false_type part;
         const bool work = nmi > 0;
-        if (work) read_frags(0, 0, 0, 0, part);
+        if (work) read_frags(0, 0, 0, part);
         for (int kt = 0; kt + 1 < nk; ++kt) {
             if (work) {
-                read_frags(kt, bs, 1, 1, part); multiply(0, part);
-                read_frags(kt, bs, 2, 0, part); multiply(1, part);
-                read_frags(kt, bs, 3, 1, part); multiply(0, part);
+                read_frags(kt, bs, 1, part); multiply(0, r0, part);
+                read_frags(kt, bs, 2, part); multiply(1, r0, part);
+                read_frags(kt, bs, 3, part); multiply(2, r0, part);
             }
             if (kt + 2 < nk) wait_dma<kDmaHalf>(); else wait_dma<0>();
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -314,39 +341,41 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             if (kt + 3 < nk) issue_b(kt + 3, bs);
             bs = next_slot(bs);
             if (work) {
-                read_frags(kt + 1, bs, 0, 0, part);
-                multiply(1, part);
+                read_frags(kt + 1, bs, 0, part);  // unit 0 of the next step lands in set 0 ...
+                multiply(3, r0, part);            // ... while unit 3 multiplies set 1 of both operands
             }
         }
         if (work) {
-            read_frags(nk - 1, bs, 1, 1, part); multiply(0, part);
-            read_frags(nk - 1, bs, 2, 0, part); multiply(1, part);
-            read_frags(nk - 1, bs, 3, 1, part); multiply(0, part);
-            multiply(1, part);
+            read_frags(nk - 1, bs, 1, part); multiply(0, r0, part);
+            read_frags(nk - 1, bs, 2, part); multiply(1, r0, part);
+            read_frags(nk - 1, bs, 3, part); multiply(2, r0, part);
+            multiply(3, r0, part);
         }
     }
 
-    // ---- epilogue.  Element v of lane l of a 32x32 accumulator sits at row 8*(v/4) + 4*(l/32) + v%4,
-    // column l%32: one column per lane.  Results are turned through LDS (free after the last stage) so
-    // that global stores are 16 bytes per lane on full 128-byte lines.
+    // ---- epilogue.  Element i of lane l of a 16x16 accumulator sits at row 4*(l/16) + i, column l%16: one
+    // column per lane.  Results are turned through LDS (free after the last stage) so that global stores
+    // are 16 bytes per lane on full 128-byte lines.
     block_barrier();  // every wave has read its last operands: the stage buffers can be reused
     if (MODE == 1) {
         // act tile [256 rows][128 columns] bf16, row pitch 272 B
         constexpr int kPitchC = 128 * 2 + 16;
         auto store_tile = [&](bool low_part) {
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) {
-                if (mi >= nmi) break;
+            for (int f = 0; f < 8; ++f) {
+                if (f >= 2 * nmi) break;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = wm * 128 + mi * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
-                    const float g = acc[mi][0][v];
-                    const float u = acc[mi][1][v];
-                    const float val = silu_mul(g, u);
-                    uint16_t bits = f32_to_bf16_bits(val);
-                    if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
-                    *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + r32) * 2) = bits;
-                }
+                for (int gg = 0; gg < 2; ++gg)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = wm * 128 + f * 16 + 4 * kq + i;
+                        const float g = acc[f][gg][i];
+                        const float u = acc[f][gg + 2][i];
+                        const float val = silu_mul(g, u);
+                        uint16_t bits = f32_to_bf16_bits(val);
+                        if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
+                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = bits;
+                    }
             }
             __syncthreads();
             uint16_t* dst = low_part ? p.act_lo : p.act;
@@ -376,11 +405,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         for (int mi = 0; mi < 4; ++mi) {
             if (mi >= nmi) break;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = 8 * (v >> 2) + 4 * kh + (v & 3);
-                *reinterpret_cast<float*>(ytile + row * kPitchY + r32 * 4) = acc[mi][0][v];
-                *reinterpret_cast<float*>(ytile + row * kPitchY + (32 + r32) * 4) = acc[mi][1][v];
-            }
+            for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = hh * 16 + 4 * kq + i;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        *reinterpret_cast<float*>(ytile + row * kPitchY + (g * 16 + r16) * 4) = acc[mi * 2 + hh][g][i];
+                }
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
             for (int it = 0; it < 8; ++it) {
