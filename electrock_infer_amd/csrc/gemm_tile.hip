@@ -243,8 +243,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         for (int j = 0; j < 4; ++j)
             if (FULL || h * 4 + j < 2 * nmi) {
 #pragma unroll
-                for (int g = 0; g < 4; ++g)
+                for (int gi = 0; gi < 4; ++gi) {
+                    const int g = (j & 1) ? 3 - gi : gi;  // serpentine: one operand changes between neighbours
                     acc[h * 4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[h][j], fb[k32][g], acc[h * 4 + j][g], 0, 0, 0);
+                }
             }
         if (FULL) {
 #pragma unroll
@@ -297,7 +299,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             // (weight fragment 0 and token fragment 0 first: the next unit starts with them)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                acc[4 + (i >> 2)][i & 3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][i >> 2], fb[1][i & 3], acc[4 + (i >> 2)][i & 3], 0, 0, 0);
+                const int j = i >> 2, g = (j & 1) ? 3 - (i & 3) : (i & 3);  // serpentine, as in multiply()
+                acc[4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][j], fb[1][g], acc[4 + j][g], 0, 0, 0);
                 const int n = i >> 1;
                 if ((i & 1) == 0) {
                     if (n < 4) { if (CA) copy_a(n, kt + 2); } else { if (CB) copy_b(n - 4, kt + 3, bs); }
