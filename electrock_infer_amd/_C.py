@@ -96,3 +96,36 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
         sorted_token_ids.data_ptr(), sorted_token_ids.numel(), expert_ids.data_ptr(), expert_ids.numel(),
         num_tokens_post_pad.data_ptr(), _lib.current_stream(topk_ids.device))
     _lib.check(code, "moe_align_block_size")
+
+
+def _norm_args(input: torch.Tensor, weight: torch.Tensor):
+    hidden = input.size(-1)
+    if weight.numel() != hidden:
+        raise RuntimeError("weight must be [hidden_size]")
+    if weight.dtype not in (input.dtype, torch.float32):
+        raise RuntimeError("weight must have the input's dtype or float32")
+    return hidden, (input.numel() // hidden if hidden else 0)
+
+
+def rms_norm(input: torch.Tensor, epsilon: float, weight: torch.Tensor) -> None:
+    """In-place RMSNorm with the native op's rounding: input = T((input * weight) * rsqrt(mean(input^2) + eps))
+    (pytorch_bind.cpp:53-58, src/add_rms_norm.hip:87-140)."""
+    _lib.require_device(input, weight)
+    hidden, rows = _norm_args(input, weight)
+    code = _lib.load().em_rms_norm(input.data_ptr(), input.data_ptr(), weight.data_ptr(), rows, hidden, float(epsilon),
+                                   _lib.dtype_code(input.dtype), _lib.dtype_code(weight.dtype), _lib.NORM_OP,
+                                   _lib.current_stream(input.device))
+    _lib.check(code, "rms_norm")
+
+
+def add_rms_norm(input: torch.Tensor, residual: torch.Tensor, epsilon: float, weight: torch.Tensor) -> None:
+    """In place: residual = T(input + residual); input = T((residual * weight) * rsqrt(mean(residual^2) + eps))
+    (pytorch_bind.cpp:60-66, src/add_rms_norm.hip:24-84)."""
+    _lib.require_device(input, residual, weight)
+    hidden, rows = _norm_args(input, weight)
+    if residual.shape != input.shape or residual.dtype != input.dtype:
+        raise RuntimeError("residual must match input")
+    code = _lib.load().em_add_rms_norm(input.data_ptr(), residual.data_ptr(), input.data_ptr(), residual.data_ptr(),
+                                       weight.data_ptr(), rows, hidden, float(epsilon), _lib.dtype_code(input.dtype),
+                                       _lib.dtype_code(weight.dtype), _lib.NORM_OP, _lib.current_stream(input.device))
+    _lib.check(code, "add_rms_norm")

@@ -13,6 +13,8 @@ from ._build import LIB_PATH
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 ITYPE_I32, ITYPE_I64 = 0, 1
 
+NORM_LAYER, NORM_OP = 0, 1   # rounding points of layers/layernorm.py resp. of the native add_rms_norm op
+
 FLAG_OUT_F32 = 1 << 0
 FLAG_ACCURATE = 1 << 1
 FLAG_GATE_F32_LOGITS = 1 << 2
@@ -27,7 +29,7 @@ FLAG_FORCE_GENERIC = 1 << 16
 EXPORTED_SYMBOLS = (
     "em_version", "em_error_string", "em_topk_softmax", "em_moe_align_block_size",
     "em_silu_and_mul", "em_moe_sum", "em_moe_workspace_bytes", "em_moe_workspace_layout",
-    "em_moe_forward", "em_moe_forward_gated", "em_gate_topk_softmax",
+    "em_moe_forward", "em_moe_forward_gated", "em_gate_topk_softmax", "em_rms_norm", "em_add_rms_norm",
 )
 
 
@@ -75,6 +77,10 @@ def load() -> ctypes.CDLL:
     lib.em_moe_forward_gated.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
     lib.em_gate_topk_softmax.restype = i32
     lib.em_gate_topk_softmax.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.em_rms_norm.restype = i32
+    lib.em_rms_norm.argtypes = [vp, vp, vp, i64, i32, ctypes.c_double, i32, i32, i32, vp]
+    lib.em_add_rms_norm.restype = i32
+    lib.em_add_rms_norm.argtypes = [vp, vp, vp, vp, vp, i64, i32, ctypes.c_double, i32, i32, i32, vp]
     _lib = lib
     return lib
 

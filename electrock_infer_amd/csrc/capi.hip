@@ -113,6 +113,30 @@ int em_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dt
     return launch_moe_sum(in, out, T, topk, H, dtype, as_stream(stream));
 }
 
+int em_rms_norm(const void* x_in, void* x_out, const void* weight, int64_t T, int H, double eps, int dtype,
+                int weight_dtype, int semantics, void* stream) {
+    if (T < 0 || H <= 0 || T >= (int64_t(1) << 31)) return EM_ERR_BAD_SHAPE;
+    if (!dtype_ok(dtype) || !dtype_ok(weight_dtype)) return EM_ERR_BAD_DTYPE;
+    if (semantics != EM_NORM_LAYER && semantics != EM_NORM_OP) return EM_ERR_BAD_SHAPE;
+    if (!rms_norm_supported(H, dtype, weight_dtype)) return EM_ERR_UNSUPPORTED;
+    if (T == 0) return 0;
+    if (!x_in || !x_out || !weight) return EM_ERR_NULL_POINTER;
+    return launch_rms_norm(x_in, nullptr, weight, x_out, nullptr, T, H, static_cast<float>(eps), dtype, weight_dtype,
+                           semantics == EM_NORM_LAYER, as_stream(stream));
+}
+
+int em_add_rms_norm(const void* x_in, const void* residual_in, void* x_out, void* residual_out, const void* weight,
+                    int64_t T, int H, double eps, int dtype, int weight_dtype, int semantics, void* stream) {
+    if (T < 0 || H <= 0 || T >= (int64_t(1) << 31)) return EM_ERR_BAD_SHAPE;
+    if (!dtype_ok(dtype) || !dtype_ok(weight_dtype)) return EM_ERR_BAD_DTYPE;
+    if (semantics != EM_NORM_LAYER && semantics != EM_NORM_OP) return EM_ERR_BAD_SHAPE;
+    if (!rms_norm_supported(H, dtype, weight_dtype)) return EM_ERR_UNSUPPORTED;
+    if (T == 0) return 0;
+    if (!x_in || !residual_in || !x_out || !residual_out || !weight) return EM_ERR_NULL_POINTER;
+    return launch_rms_norm(x_in, residual_in, weight, x_out, residual_out, T, H, static_cast<float>(eps), dtype,
+                           weight_dtype, semantics == EM_NORM_LAYER, as_stream(stream));
+}
+
 int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_layout* L) {
     if (!L) return EM_ERR_NULL_POINTER;
     if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;

@@ -90,6 +90,10 @@ int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  hipStream_t s);
 int launch_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, hipStream_t s);
 int launch_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype, hipStream_t s);
+bool rms_norm_supported(int H, int dtype, int weight_dtype);
+// res_in == nullptr: plain RMSNorm; x_out / res_out may alias their inputs
+int launch_rms_norm(const void* x_in, const void* res_in, const void* weight, void* x_out, void* res_out,
+                    int64_t T, int H, float eps, int dtype, int weight_dtype, bool layer_semantics, hipStream_t s);
 
 // Problem description shared by the expert GEMM stages.
 struct MoeProblem {

@@ -143,6 +143,38 @@ int em_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtyp
 int em_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype,
                void* stream);
 
+/* Rounding points of the two RMSNorm definitions the reference holds (T = rounding to the element type):
+ *   EM_NORM_LAYER  layers/layernorm.py:17-41, what the model runs:
+ *                  s = f32(x) + f32(residual); residual' = T(s); var = mean(s^2);
+ *                  y = T( f32(T(s * rsqrt(var + eps))) * f32(weight) )
+ *   EM_NORM_OP     src/add_rms_norm.hip:24-84,87-140, the native op:
+ *                  r = T(x + residual); residual' = r; var = mean(f32(r)^2);
+ *                  y = T( (f32(r) * f32(weight)) * rsqrt(var + eps) )
+ */
+#define EM_NORM_LAYER 0
+#define EM_NORM_OP 1
+
+/*
+ * RMSNorm over the last dimension of x [T, H]; x_out may be x_in.
+ * Replaces  _C.rms_norm(input, epsilon, weight)  (pytorch_bind.cpp:53-58, src/include/ops.h:31-34)
+ * and RMSNorm.rms_forward (layers/layernorm.py:17-27).
+ *   dtype in {F32, BF16, F16}; weight [H] of the same dtype or F32; H a multiple of 8 (4 for F32),
+ *   at most 16384 (8192 for F32), else EM_ERR_UNSUPPORTED.
+ */
+int em_rms_norm(const void* x_in, void* x_out, const void* weight, int64_t T, int H, double eps,
+                int dtype, int weight_dtype, int semantics, void* stream);
+
+/*
+ * Residual add + RMSNorm: x_out = norm(x_in + residual_in) * weight, residual_out = x_in + residual_in;
+ * outputs may alias their inputs (the native op works in place).
+ * Replaces  _C.add_rms_norm(input, residual, epsilon, weight)
+ *   (pytorch_bind.cpp:60-66, src/include/ops.h:36-40) and RMSNorm.add_rms_forward
+ *   (layers/layernorm.py:29-41), the step in front of the MoE block (models/mixtral.py:194-197).
+ */
+int em_add_rms_norm(const void* x_in, const void* residual_in, void* x_out, void* residual_out,
+                    const void* weight, int64_t T, int H, double eps, int dtype, int weight_dtype,
+                    int semantics, void* stream);
+
 /*
  * Bytes of device workspace em_moe_forward needs for these shapes
  * (0 for invalid shapes).  The workspace must be 256-byte aligned.

@@ -16,6 +16,10 @@ means:
                             reference's own test restated in pure Python
                             (moe_align_block_size_loop), structural invariants
   silu_and_mul / moe_sum    torch.nn.functional.silu / torch.sum library routines
+  gate_logits               hand-worked case, torch.nn.functional.linear in float64
+  rms_norm                  the reference's own torch op chains run by the library, exact small
+                            cases, power-of-two scale invariance, a case where the two rounding
+                            conventions differ
   moe_layer_fp32            dense all-experts formulation with torch.topk routing,
                             one-hot routing reducing to a plain SwiGLU MLP
   moe_layer_staged_bf16     its rounding points against moe_layer_fp32 within
@@ -64,6 +68,59 @@ def gate_logits(x: np.ndarray, gate_w: np.ndarray, round_bf16: bool = True) -> n
     acc = np.asarray(x, dtype=np.float64) @ np.asarray(gate_w, dtype=np.float64).T
     out = acc.astype(np.float32)
     return to_bf16_f32(out) if round_bf16 else out
+
+
+# ----------------------------------------------------------------------------
+# the step in front of the MoE block: RMSNorm, optionally with the residual add
+# ----------------------------------------------------------------------------
+def round_to(a: np.ndarray, dtype: str) -> np.ndarray:
+    """Round float32 values to the element type ("float32", "bfloat16", "float16"), returned as float32."""
+    a = np.asarray(a, dtype=np.float32)
+    if dtype == "bfloat16":
+        return to_bf16_f32(a)
+    if dtype == "float16":
+        return a.astype(np.float16).astype(np.float32)
+    if dtype == "float32":
+        return a
+    raise ValueError(dtype)
+
+
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float, residual: np.ndarray = None,
+             semantics: str = "layer", dtype: str = "bfloat16"):
+    """RMSNorm over the last axis, with the residual add when ``residual`` is given.
+
+    x, residual [T, H] and weight [H] hold values of tensors of element type ``dtype`` (weight may also be
+    float32) as float32 arrays.  Returns y, or (y, residual_out), as float32 arrays of ``dtype`` values.
+
+    semantics "layer" -- what the model runs (layers/layernorm.py:17-41): the sum x + residual and its mean
+    square stay float32; residual_out = T(sum); the normalised value is rounded to T before and after the
+    multiplication by the weight.
+    semantics "op" -- the native op (src/add_rms_norm.hip:47-52,76-80 and 103-106,130-133): the sum is
+    rounded to T first and everything else uses the rounded value; one rounding of (value * weight) * rstd.
+
+    The mean of squares is accumulated in float64 and rounded once to float32 (the reference sums in
+    float32 in an order of its library's choosing); rsqrt is 1 / sqrt in float32.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    w = np.asarray(weight, dtype=np.float32)
+    one = np.float32(1.0)
+    res_out = None
+    if residual is not None:
+        s = x + np.asarray(residual, dtype=np.float32)      # float32 add
+        res_out = round_to(s, dtype)
+        if semantics == "op":
+            s = res_out
+    else:
+        s = x
+    var = (s.astype(np.float64) ** 2).mean(axis=-1, keepdims=True).astype(np.float32)
+    rstd = one / np.sqrt(var + np.float32(eps), dtype=np.float32)
+    if semantics == "layer":
+        y = round_to(round_to(s * rstd, dtype) * w, dtype)
+    elif semantics == "op":
+        y = round_to((s * w) * rstd, dtype)
+    else:
+        raise ValueError(semantics)
+    return y if residual is None else (y, res_out)
 
 
 # ----------------------------------------------------------------------------

@@ -263,3 +263,121 @@ def test_golden_fixture_c1():
     assert np.array_equal(n, gold["num_tokens_post_pad"])
     out = O.moe_layer_fp32(x, lg, w13, w2).numpy()
     np.testing.assert_allclose(out, gold["out"], rtol=1e-4, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------
+# RMSNorm (the step in front of the MoE block)
+# ----------------------------------------------------------------------------
+_TORCH_DT = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
+
+
+def _ulp(v, dtype):
+    bits = {"float32": 23, "bfloat16": 7, "float16": 10}[dtype]
+    return 2.0 ** (np.floor(np.log2(np.maximum(np.abs(v), 2.0 ** -14))) - bits)
+
+
+def _layer_chain(x, residual, weight, eps):
+    """The reference module's own op chains (layers/layernorm.py:17-41), run by torch on the CPU."""
+    orig = x.dtype
+    if residual is None:
+        xf = x.to(torch.float32)
+        var = xf.pow(2).mean(dim=-1, keepdim=True)
+        xf = xf * torch.rsqrt(var + eps)
+        return xf.to(orig).mul_(weight), None
+    xf = x.to(torch.float32).add_(residual.to(torch.float32))
+    res = xf.to(orig)
+    var = xf.pow(2).mean(dim=-1, keepdim=True)
+    xf = xf * torch.rsqrt(var + eps)
+    return xf.to(orig).mul_(weight), res
+
+
+def _op_chain(x, residual, weight, eps):
+    """The native op's arithmetic (src/add_rms_norm.hip:47-52,76-80) written with torch library ops."""
+    r = x if residual is None else (x + residual)           # add in the element type: one rounding
+    var = r.to(torch.float32).pow(2).mean(dim=-1, keepdim=True)
+    y = (r.to(torch.float32) * weight.to(torch.float32) * torch.rsqrt(var + eps)).to(x.dtype)
+    return y, (None if residual is None else r)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
+@pytest.mark.parametrize("semantics", ["layer", "op"])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_rms_norm_matches_the_references_torch_chains(dtype, semantics, with_residual):
+    g = torch.Generator().manual_seed(5)
+    T, H, eps = 37, 512, 1e-5
+    x = torch.randn(T, H, generator=g).to(_TORCH_DT[dtype])
+    res = torch.randn(T, H, generator=g).to(_TORCH_DT[dtype]) if with_residual else None
+    w = (1.0 + 0.1 * torch.randn(H, generator=g)).to(_TORCH_DT[dtype])
+    chain = _layer_chain if semantics == "layer" else _op_chain
+    y_ref, res_ref = chain(x.clone(), None if res is None else res.clone(), w, eps)
+    out = O.rms_norm(x.float().numpy(), w.float().numpy(), eps, None if res is None else res.float().numpy(),
+                     semantics=semantics, dtype=dtype)
+    y, res_out = (out, None) if res is None else out
+    if with_residual:
+        np.testing.assert_array_equal(res_out, res_ref.float().numpy())       # one float32 add, one rounding: exact
+    # the variance is summed in a different order (float64 here, float32 in the library): the results may sit on
+    # neighbouring values of the element type where a product falls next to a rounding boundary
+    if dtype == "float32":   # nothing is rounded to a coarser type: a few float32 steps from rstd and the products
+        np.testing.assert_allclose(y, y_ref.numpy(), rtol=6e-7, atol=1e-9)
+        return
+    err = np.abs(y - y_ref.float().numpy())
+    assert (err <= _ulp(y_ref.float().numpy(), dtype) * 1.0001).all()
+    assert (err > 0).mean() < 0.01
+
+
+def test_rms_norm_exact_small_cases():
+    # var = 4, rstd = 1/2 exactly: y = w
+    w = np.array([1.0, 2.0, 0.5, -1.0], dtype=np.float32)
+    y = O.rms_norm(np.full((1, 4), 2.0, np.float32), w, 0.0)
+    np.testing.assert_array_equal(y, w[None])
+    # residual add first: 1 + 1 = 2, same result, residual_out = 2
+    for sem in ("layer", "op"):
+        y, r = O.rms_norm(np.ones((1, 4), np.float32), w, 0.0, np.ones((1, 4), np.float32), semantics=sem)
+        np.testing.assert_array_equal(y, w[None])
+        np.testing.assert_array_equal(r, np.full((1, 4), 2.0, np.float32))
+    # eps matters: x = 0 gives 0, not NaN, as long as eps > 0
+    assert np.all(O.rms_norm(np.zeros((2, 8), np.float32), np.ones(8, np.float32), 1e-5) == 0.0)
+    # 3-4-5: mean square of (3, 4) is 12.5; y = x / sqrt(12.5) in float32
+    y = O.rms_norm(np.array([[3.0, 4.0]], np.float32), np.ones(2, np.float32), 0.0, dtype="float32")
+    np.testing.assert_allclose(y, np.array([[3.0, 4.0]]) / np.sqrt(12.5), rtol=2e-7)
+
+
+@pytest.mark.parametrize("semantics", ["layer", "op"])
+def test_rms_norm_power_of_two_scale_invariance(semantics):
+    # with eps = 0 a scaling of the input by 2^k changes nothing, bit for bit; a scaling of the weight scales the output
+    rng = np.random.default_rng(3)
+    x = O.to_bf16_f32(rng.standard_normal((9, 256)).astype(np.float32))
+    r = O.to_bf16_f32(rng.standard_normal((9, 256)).astype(np.float32))
+    w = O.to_bf16_f32((1 + 0.1 * rng.standard_normal(256)).astype(np.float32))
+    y0, r0 = O.rms_norm(x, w, 0.0, r, semantics=semantics)
+    y1, r1 = O.rms_norm(x * 8, w, 0.0, r * 8, semantics=semantics)
+    np.testing.assert_array_equal(y0, y1)
+    np.testing.assert_array_equal(r0 * 8, r1)
+    y2, _ = O.rms_norm(x, w * 4, 0.0, r, semantics=semantics)
+    np.testing.assert_array_equal(y0 * 4, y2)
+    # unit weight: every row of the (float32) result has mean square 1
+    y = O.rms_norm(x, np.ones(256, np.float32), 0.0, dtype="float32")
+    np.testing.assert_allclose((y.astype(np.float64) ** 2).mean(-1), 1.0, rtol=1e-6)
+
+
+def test_rms_norm_rounding_conventions_differ_where_expected():
+    # x + residual = 1 + 2^-8 is not a bf16 value: the layer keeps it for the variance and the product, the op
+    # rounds it to 1 first
+    x = np.array([[1.0, 3.0]], np.float32)
+    r = np.array([[2.0 ** -8, 0.0]], np.float32)
+    w = np.ones(2, np.float32)
+    (yl, rl), (yo, ro) = (O.rms_norm(x, w, 0.0, r, semantics=s, dtype="float32") for s in ("layer", "op"))
+    np.testing.assert_array_equal(rl, x + r)          # float32 element type: nothing is rounded
+    (ylb, rlb), (yob, rob) = (O.rms_norm(x, w, 0.0, r, semantics=s, dtype="bfloat16") for s in ("layer", "op"))
+    np.testing.assert_array_equal(rlb, np.array([[1.0, 3.0]], np.float32))   # both return the rounded sum
+    np.testing.assert_array_equal(rob, rlb)
+    # layer: var = ((1 + 2^-8)^2 + 9) / 2 ; op: var = (1 + 9) / 2 = 5 exactly
+    np.testing.assert_allclose(yob[0, 1], O.to_bf16_f32(np.float32(3.0 / np.sqrt(5.0))), rtol=0)
+    # double against single rounding: s * rstd = 1 + 2^-8 (a tie, rounds to 1), weight 1.5
+    s = np.array([[1.0 + 2.0 ** -8, 1.0 + 2.0 ** -8]], np.float32)
+    eps = float(np.float32(1.0) - (s.astype(np.float64) ** 2).mean().astype(np.float32))  # makes var + eps = 1
+    w15 = np.full(2, 1.5, np.float32)
+    yl2 = O.rms_norm(s, w15, eps, dtype="bfloat16", semantics="layer")
+    yo2 = O.rms_norm(s, w15, eps, dtype="bfloat16", semantics="op")
+    np.testing.assert_array_equal(yl2, np.full((1, 2), 1.5, np.float32))          # T(T(1.0039) * 1.5) = 1.5
+    np.testing.assert_array_equal(yo2, np.full((1, 2), 1.5078125, np.float32))    # T(1.0039 * 1.5) = 1.5078125
