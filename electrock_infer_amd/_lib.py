@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "em_version", "em_error_string", "em_topk_softmax", "em_moe_align_block_size",
     "em_silu_and_mul", "em_moe_sum", "em_moe_workspace_bytes", "em_moe_workspace_layout",
     "em_moe_forward", "em_moe_forward_gated", "em_gate_topk_softmax", "em_rms_norm", "em_add_rms_norm",
+    "em_norm_gate_topk_softmax", "em_moe_forward_normed",
 )
 
 
@@ -81,6 +82,12 @@ def load() -> ctypes.CDLL:
     lib.em_rms_norm.argtypes = [vp, vp, vp, i64, i32, ctypes.c_double, i32, i32, i32, vp]
     lib.em_add_rms_norm.restype = i32
     lib.em_add_rms_norm.argtypes = [vp, vp, vp, vp, vp, i64, i32, ctypes.c_double, i32, i32, i32, vp]
+    lib.em_norm_gate_topk_softmax.restype = i32
+    lib.em_norm_gate_topk_softmax.argtypes = [vp, vp, vp, i32, ctypes.c_double, i32, vp, vp, vp, i64, i32, i32, i32, i32,
+                                              i32, vp, vp, vp, vp]
+    lib.em_moe_forward_normed.restype = i32
+    lib.em_moe_forward_normed.argtypes = [vp, vp, vp, i32, ctypes.c_double, i32, vp, vp, vp, vp, vp, vp, i64, i32, i32,
+                                          i32, i32, i32, vp, sz, u32, vp]
     _lib = lib
     return lib
 

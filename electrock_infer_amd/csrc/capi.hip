@@ -176,11 +176,24 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k) {
 
 namespace {
 
-// The layer behind both entry points: the routing comes either from caller-provided logits or from the
-// gate matrix (gate_w != nullptr: logits = x . gate_w^T computed in the router's launch).
+// RMSNorm in front of the block: x of the layer is then the buffer the normalised rows are written to
+struct NormFront {
+    const void* x_in;
+    const void* residual_in;  // may be null: plain RMSNorm
+    const void* weight;
+    int weight_dtype;
+    float eps;
+    bool layer_semantics;
+    void* residual_out;
+};
+
+// The layer behind the entry points: the routing comes either from caller-provided logits or from the
+// gate matrix (gate_w != nullptr: logits = x . gate_w^T computed in the router's launch), which may have
+// the RMSNorm of the rows in front (norm != nullptr: that launch also writes x).
 int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype, const void* gate_w, const void* w13,
                      const void* w2, void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
-                     void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+                     void* workspace, size_t workspace_bytes, unsigned flags, void* stream,
+                     const NormFront* norm = nullptr) {
     if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
     if (gate_w == nullptr && !dtype_ok(logits_dtype)) return EM_ERR_BAD_DTYPE;
     if (gate_w != nullptr && !gate_router_supported(H, E)) return EM_ERR_UNSUPPORTED;
@@ -226,10 +239,15 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.ksplit = static_cast<int>(L.ksplit);
 
     if (!(flags & EM_FLAG_SKIP_ROUTER)) {
-        rc = gate_w != nullptr
-                 ? launch_gate_router(x, gate_w, T, H, E, top_k, renormalize, (flags & EM_FLAG_GATE_F32_LOGITS) ? 0 : 1,
-                                      nullptr, topk_w, topk_ids, s)
-                 : launch_router(router_logits, logits_dtype, T, E, top_k, renormalize, topk_w, topk_ids, s);
+        const int round_logits = (flags & EM_FLAG_GATE_F32_LOGITS) ? 0 : 1;
+        if (norm != nullptr)
+            rc = launch_norm_gate_router(norm->x_in, norm->residual_in, norm->weight, norm->weight_dtype, norm->eps,
+                                         norm->layer_semantics, const_cast<void*>(x), norm->residual_out, gate_w, T, H,
+                                         E, top_k, renormalize, round_logits, nullptr, topk_w, topk_ids, s);
+        else if (gate_w != nullptr)
+            rc = launch_gate_router(x, gate_w, T, H, E, top_k, renormalize, round_logits, nullptr, topk_w, topk_ids, s);
+        else
+            rc = launch_router(router_logits, logits_dtype, T, E, top_k, renormalize, topk_w, topk_ids, s);
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_ALIGN)) {
@@ -288,6 +306,48 @@ int em_moe_forward_gated(const void* x, const void* gate_w, const void* w13, con
     if (!gate_w && T > 0 && shapes_ok(T, H, I, E, top_k)) return EM_ERR_NULL_POINTER;
     return moe_forward_impl(x, nullptr, EM_DTYPE_BF16, gate_w, w13, w2, out, T, H, I, E, top_k, renormalize, workspace,
                             workspace_bytes, flags, stream);
+}
+
+int em_moe_forward_normed(const void* x_in, const void* residual_in, const void* norm_weight, int norm_weight_dtype,
+                          double eps, int semantics, void* h_buf, void* residual_out, const void* gate_w,
+                          const void* w13, const void* w2, void* out, int64_t T, int H, int I, int E, int top_k,
+                          int renormalize, void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
+    if (norm_weight_dtype != EM_DTYPE_BF16 && norm_weight_dtype != EM_DTYPE_F32) return EM_ERR_BAD_DTYPE;
+    if (semantics != EM_NORM_LAYER && semantics != EM_NORM_OP) return EM_ERR_BAD_SHAPE;
+    if (T == 0) return 0;
+    if (!x_in || !norm_weight || !h_buf || !gate_w || (residual_in && !residual_out)) return EM_ERR_NULL_POINTER;
+    if (!aligned(x_in, 16) || !aligned(norm_weight, 16) || (residual_in && !aligned(residual_in, 16)) ||
+        (residual_out && !aligned(residual_out, 16)))
+        return EM_ERR_ALIGNMENT;
+    // the rows are read twice: the new residual must not land on either input
+    if (residual_in && (residual_out == residual_in || residual_out == x_in || h_buf == residual_in))
+        return EM_ERR_UNSUPPORTED;
+    const NormFront norm{x_in, residual_in, norm_weight, norm_weight_dtype, static_cast<float>(eps),
+                         semantics == EM_NORM_LAYER, residual_out};
+    return moe_forward_impl(h_buf, nullptr, EM_DTYPE_BF16, gate_w, w13, w2, out, T, H, I, E, top_k, renormalize, workspace,
+                            workspace_bytes, flags, stream, &norm);
+}
+
+int em_norm_gate_topk_softmax(const void* x_in, const void* residual_in, const void* norm_weight, int norm_weight_dtype,
+                              double eps, int semantics, void* h_out, void* residual_out, const void* gate_w, int64_t T,
+                              int H, int E, int k, int renormalize, int round_logits_bf16, void* logits_out,
+                              float* topk_weights, int32_t* topk_ids, void* stream) {
+    if (T < 0 || H <= 0 || H % 8 != 0 || E < 1 || E > kMaxExperts || k < 1 || k > E) return EM_ERR_BAD_SHAPE;
+    if (norm_weight_dtype != EM_DTYPE_BF16 && norm_weight_dtype != EM_DTYPE_F32) return EM_ERR_BAD_DTYPE;
+    if (semantics != EM_NORM_LAYER && semantics != EM_NORM_OP) return EM_ERR_BAD_SHAPE;
+    if (!gate_router_supported(H, E)) return EM_ERR_UNSUPPORTED;
+    if (T == 0) return 0;
+    if (!x_in || !norm_weight || !h_out || !gate_w || !topk_weights || !topk_ids || (residual_in && !residual_out))
+        return EM_ERR_NULL_POINTER;
+    if (!aligned(x_in, 16) || !aligned(h_out, 16) || !aligned(gate_w, 16) || !aligned(norm_weight, 16) ||
+        (residual_in && (!aligned(residual_in, 16) || !aligned(residual_out, 16))))
+        return EM_ERR_ALIGNMENT;
+    if (residual_in && (residual_out == residual_in || residual_out == x_in || h_out == residual_in))
+        return EM_ERR_UNSUPPORTED;  // the rows are read twice: the new residual must not land on either input
+    return launch_norm_gate_router(x_in, residual_in, norm_weight, norm_weight_dtype, static_cast<float>(eps),
+                                   semantics == EM_NORM_LAYER, h_out, residual_out, gate_w, T, H, E, k, renormalize,
+                                   round_logits_bf16 ? 1 : 0, logits_out, topk_weights, topk_ids, as_stream(stream));
 }
 
 int em_gate_topk_softmax(const void* x, const void* gate_w, int64_t T, int H, int E, int k, int renormalize,

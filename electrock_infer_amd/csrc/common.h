@@ -84,6 +84,12 @@ int launch_router(const void* logits, int logits_dtype, int64_t T, int E, int k,
 bool gate_router_supported(int H, int E);
 int launch_gate_router(const void* x, const void* gate_w, int64_t T, int H, int E, int k, int renorm,
                        int round_bf16, void* logits_out, float* w, int32_t* ids, hipStream_t s);
+// RMSNorm (behind a residual add when res_in != nullptr) + gate + router in one launch; bf16 rows,
+// norm weight bf16 or fp32; h_out receives the normalised rows, res_out the new residual
+int launch_norm_gate_router(const void* x_in, const void* res_in, const void* norm_w, int norm_w_dtype, float eps,
+                            bool layer_semantics, void* h_out, void* res_out, const void* gate_w, int64_t T, int H,
+                            int E, int k, int renorm, int round_bf16, void* logits_out, float* w, int32_t* ids,
+                            hipStream_t s);
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
                  int32_t* post_pad, int32_t* seg_out /* [E+1] padded segment starts, may be null */,

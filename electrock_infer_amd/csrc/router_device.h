@@ -61,4 +61,38 @@ __device__ __forceinline__ void route_from_logit(float v, int lane, int64_t t, i
     route_group<kWave>(v, lane, t, true, E, k, renorm, out_w, out_ids);
 }
 
+// Tail of the kernels that compute the logits of 16 tokens per workgroup on the MFMA, the waves splitting H:
+// `acc` is the wave's partial 16x16 tile (lane l: token l % 16, experts 4 * (l / 16) .. + 3).  The partial
+// tiles meet in LDS and are added in wave order; optional rounding to bf16 as the reference's linear does
+// (layers/linear.py:53-54); then E adjacent lanes per token run the selection, 64 / E tokens per wavefront.
+// Contains a block barrier: all waves of the workgroup must call it.
+template <int E_, int WAVES>
+__device__ __forceinline__ void reduce_tiles_and_route(f32x4_t acc, float (*partial)[16][E_], int wave, int lane,
+                                                       int64_t t0, int64_t T, int k, int renorm, int round_bf16,
+                                                       void* __restrict__ logits_out, float* __restrict__ out_w,
+                                                       int32_t* __restrict__ out_ids) {
+    const int r16 = lane & 15, kq = lane >> 4;
+    if (4 * kq < E_) *reinterpret_cast<f32x4_t*>(&partial[wave][r16][4 * kq]) = acc;
+    __syncthreads();
+    constexpr int kTokPerWave = kWave / E_;
+    if (wave * kTokPerWave < 16) {  // whole waves leave together
+        const int tok = wave * kTokPerWave + lane / E_;
+        const int e = lane % E_;
+        const int64_t t = t0 + tok;
+        const bool valid = (t < T);
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) v += partial[w][tok][e];
+        if (round_bf16) {
+            const uint16_t b = f32_to_bf16_bits(v);
+            v = bf16_bits_to_f32(b);
+            if (valid && logits_out != nullptr) static_cast<uint16_t*>(logits_out)[t * E_ + e] = b;
+        } else if (valid && logits_out != nullptr) {
+            static_cast<float*>(logits_out)[t * E_ + e] = v;
+        }
+        if (v != v) v = -INFINITY;  // a NaN logit can never be selected
+        route_group<E_>(v, lane, t, valid, E_, k, renorm, out_w, out_ids);
+    }
+}
+
 }  // namespace em

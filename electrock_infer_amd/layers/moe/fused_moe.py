@@ -208,3 +208,90 @@ def fused_experts_gated(hidden_states: torch.Tensor, gate_weight: torch.Tensor, 
         _lib.current_stream(hidden_states.device))
     _lib.check(code, "fused_experts_gated")
     return output
+
+
+def _norm_front_args(hidden_states, residual, norm_weight, gate_weight):
+    _lib.require_device(hidden_states, norm_weight, gate_weight)
+    T, H = hidden_states.shape
+    if residual is not None:
+        _lib.require_device(residual)
+        if residual.shape != hidden_states.shape or residual.dtype != hidden_states.dtype:
+            raise RuntimeError("residual must match hidden_states")
+    if norm_weight.numel() != H or norm_weight.dtype not in (torch.bfloat16, torch.float32):
+        raise RuntimeError("norm_weight must be [hidden_size], bfloat16 or float32")
+    if gate_weight.shape[1] != H:
+        raise RuntimeError("gate_weight must be [num_experts, hidden_size]")
+    if not (hidden_states.dtype == gate_weight.dtype == torch.bfloat16):
+        raise RuntimeError("the fused norm + gate computes in bfloat16: hidden_states and gate_weight must be bfloat16")
+    return T, H
+
+
+def norm_gate_topk(hidden_states: torch.Tensor, residual: Optional[torch.Tensor], norm_weight: torch.Tensor,
+                   eps: float, gate_weight: torch.Tensor, topk: int, renormalize: bool = True,
+                   bf16_logits: bool = True, return_logits: bool = False, op_rounding: bool = False):
+    """RMSNorm (behind the residual add when ``residual`` is given), router gate and router in one launch:
+    the reference's ``post_attention_layernorm`` followed by the gate and ``fused_topk``
+    (models/mixtral.py:194-197,59; layers/layernorm.py:17-41; fused_moe.py:130-164).
+
+    Returns (normed [T, H] bf16, residual_out or None, topk_weights [T, topk] fp32, topk_ids [T, topk] int32
+    [, logits [T, E]]).  ``op_rounding`` selects the native add_rms_norm op's rounding points instead of the
+    module's.
+    """
+    T, H = _norm_front_args(hidden_states, residual, norm_weight, gate_weight)
+    E = gate_weight.shape[0]
+    dev = hidden_states.device
+    normed = torch.empty_like(hidden_states)
+    res_out = torch.empty_like(hidden_states) if residual is not None else None
+    topk_weights = torch.empty(T, topk, dtype=torch.float32, device=dev)
+    topk_ids = torch.empty(T, topk, dtype=torch.int32, device=dev)
+    logits = torch.empty(T, E, dtype=torch.bfloat16 if bf16_logits else torch.float32, device=dev) if return_logits else None
+    code = _lib.load().em_norm_gate_topk_softmax(
+        hidden_states.data_ptr(), residual.data_ptr() if residual is not None else None, norm_weight.data_ptr(),
+        _lib.dtype_code(norm_weight.dtype), float(eps), _lib.NORM_OP if op_rounding else _lib.NORM_LAYER,
+        normed.data_ptr(), res_out.data_ptr() if res_out is not None else None, gate_weight.data_ptr(), T, H, E, topk,
+        1 if renormalize else 0, 1 if bf16_logits else 0, logits.data_ptr() if logits is not None else None,
+        topk_weights.data_ptr(), topk_ids.data_ptr(), _lib.current_stream(dev))
+    _lib.check(code, "norm_gate_topk")
+    out = (normed, res_out, topk_weights, topk_ids)
+    return out + (logits,) if return_logits else out
+
+
+def fused_experts_normed(hidden_states: torch.Tensor, residual: Optional[torch.Tensor], norm_weight: torch.Tensor,
+                         eps: float, gate_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk: int,
+                         renormalize: bool = True, out_dtype: Optional[torch.dtype] = None, accurate: bool = False,
+                         bf16_logits: bool = True, op_rounding: bool = False, flags: int = 0,
+                         workspace: Optional[MoeWorkspace] = None):
+    """The tail of the reference's decoder layer in one call (models/mixtral.py:194-197):
+    ``h, residual = post_attention_layernorm(hidden_states, residual); out = block_sparse_moe(h)``.
+    Returns (out [T, H], residual_out or None)."""
+    T, H = _norm_front_args(hidden_states, residual, norm_weight, gate_weight)
+    _lib.require_device(w1, w2)
+    E, two_i, Hw = w1.shape
+    I = two_i // 2
+    if Hw != H or tuple(w2.shape) != (E, H, I) or two_i != 2 * I or tuple(gate_weight.shape) != (E, H):
+        raise RuntimeError("weight shapes do not match hidden_states")
+    if not (w1.dtype == w2.dtype == torch.bfloat16):
+        raise RuntimeError("the fused MoE path computes in bfloat16: w1 and w2 must be bfloat16")
+    if accurate:
+        flags |= _lib.FLAG_ACCURATE
+    if not bf16_logits:
+        flags |= _lib.FLAG_GATE_F32_LOGITS
+    dev = hidden_states.device
+    h_buf = torch.empty_like(hidden_states)
+    res_out = torch.empty_like(hidden_states) if residual is not None else None
+    if out_dtype == torch.float32:
+        output = torch.empty((T, H), dtype=torch.float32, device=dev)
+        flags |= _lib.FLAG_OUT_F32
+    else:
+        output = h_buf          # the experts' result overwrites the normalised rows, as the reference's in-place layer does
+    if T == 0:
+        return output, res_out
+    ws = workspace or get_workspace(dev, T, H, I, E, topk)
+    code = _lib.load().em_moe_forward_normed(
+        hidden_states.data_ptr(), residual.data_ptr() if residual is not None else None, norm_weight.data_ptr(),
+        _lib.dtype_code(norm_weight.dtype), float(eps), _lib.NORM_OP if op_rounding else _lib.NORM_LAYER,
+        h_buf.data_ptr(), res_out.data_ptr() if res_out is not None else None, gate_weight.data_ptr(), w1.data_ptr(),
+        w2.data_ptr(), output.data_ptr(), T, H, I, E, topk, 1 if renormalize else 0, ws.buffer.data_ptr(),
+        ctypes.c_size_t(ws.buffer.numel()), flags, _lib.current_stream(dev))
+    _lib.check(code, "fused_experts_normed")
+    return output, res_out

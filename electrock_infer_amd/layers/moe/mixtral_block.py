@@ -7,7 +7,8 @@ import torch
 import torch.distributed as dist
 import torch.nn as nn
 
-from .fused_moe import fused_experts_gated
+from ..layernorm import RMSNorm
+from .fused_moe import fused_experts_gated, fused_experts_normed
 from .mixtral_moe import FusedMoE
 
 
@@ -60,3 +61,29 @@ class MixtralMoE(nn.Module):
         if e.reduce_results and e.tp_size > 1:
             dist.all_reduce(out)
         return out.view(orig_shape)
+
+
+class PostAttentionMoE(nn.Module):
+    """The tail of the reference's decoder layer (models/mixtral.py:194-197) as one module and one library call:
+
+        hidden_states, residual = post_attention_layernorm(hidden_states, residual)
+        hidden_states = block_sparse_moe(hidden_states)
+
+    ``forward(hidden_states, residual)`` returns ``(hidden_states, residual)`` like those two lines; the norm,
+    the gate and the router run in one launch.  Holds the reference's sub-modules under their names."""
+
+    def __init__(self, post_attention_layernorm: RMSNorm, block_sparse_moe: MixtralMoE):
+        super().__init__()
+        self.post_attention_layernorm = post_attention_layernorm
+        self.block_sparse_moe = block_sparse_moe
+
+    def forward(self, hidden_states: torch.Tensor, residual: torch.Tensor):
+        norm, moe = self.post_attention_layernorm, self.block_sparse_moe
+        e = moe.experts
+        orig_shape = hidden_states.shape
+        out, res = fused_experts_normed(hidden_states.view(-1, moe.hidden_size), residual.view(-1, moe.hidden_size),
+                                        norm.weight, norm.eps, moe.gate.weight, e.w13_weight, e.w2_weight, topk=e.top_k,
+                                        renormalize=e.renormalize, bf16_logits=moe.bf16_logits)
+        if e.reduce_results and e.tp_size > 1:
+            dist.all_reduce(out)
+        return out.view(orig_shape), res.view(orig_shape)

@@ -98,6 +98,33 @@ int em_gate_topk_softmax(const void* x, const void* gate_w, int64_t T, int H, in
                          float* topk_weights, int32_t* topk_ids, void* stream);
 
 /*
+ * RMSNorm of the rows (behind a residual add when residual_in is not NULL), router gate and top-k softmax in
+ * one launch: the two lines in front of the expert GEMMs in the reference's decoder layer
+ * (models/mixtral.py:194-197: post_attention_layernorm, then block_sparse_moe -> gate, models/mixtral.py:59).
+ *   x_in, residual_in [T, H] bf16; norm_weight [H] bf16 or F32; gate_w [E, H] bf16 (E of 8 or 16);
+ *   h_out [T, H] bf16 receives the normalised rows (the input of the experts), residual_out [T, H] bf16 the
+ *   sum x_in + residual_in.  h_out may be x_in; residual_out must be a buffer of its own (the rows are read
+ *   twice), else EM_ERR_UNSUPPORTED.  semantics: EM_NORM_LAYER / EM_NORM_OP.
+ *   logits_out may be NULL; else [T, E] bf16 (round_logits_bf16) or F32.
+ */
+int em_norm_gate_topk_softmax(const void* x_in, const void* residual_in, const void* norm_weight,
+                              int norm_weight_dtype, double eps, int semantics, void* h_out,
+                              void* residual_out, const void* gate_w, int64_t T, int H, int E, int k,
+                              int renormalize, int round_logits_bf16, void* logits_out,
+                              float* topk_weights, int32_t* topk_ids, void* stream);
+
+/*
+ * em_moe_forward_gated with that launch in front: (x_in, residual_in) -> out = MoE(norm(x_in + residual_in)),
+ * residual_out = x_in + residual_in.  h_buf [T, H] bf16 is scratch for the normalised rows (it may be x_in,
+ * and out may be h_buf); everything else as em_moe_forward_gated.
+ */
+int em_moe_forward_normed(const void* x_in, const void* residual_in, const void* norm_weight,
+                          int norm_weight_dtype, double eps, int semantics, void* h_buf, void* residual_out,
+                          const void* gate_w, const void* w13, const void* w2, void* out, int64_t T, int H,
+                          int I, int E, int top_k, int renormalize, void* workspace, size_t workspace_bytes,
+                          unsigned flags, void* stream);
+
+/*
  * Expert sort with padding to the GEMM block size.
  * Replaces  _C.moe_align_block_size(topk_ids, num_experts, block_size,
  *                                   sorted_token_ids, expert_ids, num_tokens_post_pad)
