@@ -70,16 +70,19 @@ __global__ __launch_bounds__(kGateThreads) void gate_router_kernel(
 // GEMMs and feeds them to the MFMA as it goes.  RESIDENT (H <= 4096): a lane keeps its 128 values of the
 // summed rows in registers between the two passes; else the rows are read a second time, out of L2.
 // Rounding points as in norm.hip (LAYER: the module's, else the native op's).  bf16 rows only.
-constexpr int kResidentSteps = 16;  // K steps of 32 a wave can keep in registers: 8 waves x 16 x 32 = 4096
+constexpr int kNormGateWaves = 16;   // 1024 threads: 64 kept values per lane leave room for four waves per SIMD
+constexpr int kNormGateThreads = kNormGateWaves * kWave;
+constexpr int kNormBatch = 4;        // K steps whose loads are in flight together (8 would spill)
+constexpr int kResidentSteps = 8;    // K steps of 32 a wave keeps in registers: 16 waves x 8 x 32 = 4096
 template <int E_, typename WElem, bool ADD, bool LAYER, bool RESIDENT>
-__global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
+__global__ __launch_bounds__(kNormGateThreads) void norm_gate_router_kernel(
     const uint16_t* __restrict__ x_in, const uint16_t* __restrict__ res_in,
     const typename WElem::storage* __restrict__ norm_w, float eps, uint16_t* __restrict__ h_out,
     uint16_t* __restrict__ res_out, const uint16_t* __restrict__ gate_w, int64_t T, int H, int k, int renorm,
     int round_bf16, void* __restrict__ logits_out, float* __restrict__ out_w, int32_t* __restrict__ out_ids) {
     static_assert(E_ == 8 || E_ == 16, "experts sit in the 16 rows of one MFMA");
-    __shared__ __attribute__((aligned(16))) float partial[kGateWaves][kGateTokens][E_];
-    __shared__ float sumsq[kGateWaves][kGateTokens];
+    __shared__ __attribute__((aligned(16))) float partial[kNormGateWaves][kGateTokens][E_];
+    __shared__ float sumsq[kNormGateWaves][kGateTokens];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
     const int kq = lane >> 4;
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kGateTokens;
     const int nsteps = (H + 31) / 32;
-    const int per_wave = (nsteps + kGateWaves - 1) / kGateWaves;
+    const int per_wave = (nsteps + kNormGateWaves - 1) / kNormGateWaves;
     const int s_begin = wave * per_wave;
     const int s_end = (s_begin + per_wave < nsteps) ? s_begin + per_wave : nsteps;
     const bool tok_ok = (t0 + r16 < T);
@@ -117,19 +120,19 @@ __global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
     float kept[RESIDENT ? kResidentSteps : 1][8];
     float sq = 0.0f;
 #pragma unroll
-    for (int b = 0; b < (RESIDENT ? kResidentSteps / kGateBatch : 1 << 30); ++b) {
-        const int s0 = s_begin + b * kGateBatch;
+    for (int b = 0; b < (RESIDENT ? kResidentSteps / kNormBatch : 1 << 30); ++b) {
+        const int s0 = s_begin + b * kNormBatch;
         if (s0 >= s_end) break;
-        u32x4_t xa[kGateBatch], ra[kGateBatch];
+        u32x4_t xa[kNormBatch], ra[kNormBatch];
 #pragma unroll
-        for (int i = 0; i < kGateBatch; ++i) {
+        for (int i = 0; i < kNormBatch; ++i) {
             const int h = (s0 + i) * 32 + kq * 8;
             const bool ok = (s0 + i < s_end) && (h < H) && tok_ok;
             xa[i] = ok ? *reinterpret_cast<const u32x4_t*>(x_in + row + h) : u32x4_t{0u, 0u, 0u, 0u};
             if (ADD) ra[i] = ok ? *reinterpret_cast<const u32x4_t*>(res_in + row + h) : u32x4_t{0u, 0u, 0u, 0u};
         }
 #pragma unroll
-        for (int i = 0; i < kGateBatch; ++i) {
+        for (int i = 0; i < kNormBatch; ++i) {
             const int h = (s0 + i) * 32 + kq * 8;
             const bool ok = (s0 + i < s_end) && (h < H) && tok_ok;
             float sv[8];
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
             for (int j = 0; j < 8; ++j) sq = fmaf(sv[j], sv[j], sq);
             if (RESIDENT) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) kept[b * kGateBatch + i][j] = sv[j];
+                for (int j = 0; j < 8; ++j) kept[b * kNormBatch + i][j] = sv[j];
             }
             if (ADD && ok) *reinterpret_cast<u32x4_t*>(res_out + row + h) = rounded;
         }
@@ -150,18 +153,18 @@ __global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
     __syncthreads();
     float total = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kGateWaves; ++w) total += sumsq[w][r16];
+    for (int w = 0; w < kNormGateWaves; ++w) total += sumsq[w][r16];
     const float rstd = 1.0f / sqrtf(total / static_cast<float>(H) + eps);
 
     // ---- pass 2: normalise (the rows come out of L2 this time), store, multiply with the gate rows ----
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int b = 0; b < (RESIDENT ? kResidentSteps / kGateBatch : 1 << 30); ++b) {
-        const int s0 = s_begin + b * kGateBatch;
+    for (int b = 0; b < (RESIDENT ? kResidentSteps / kNormBatch : 1 << 30); ++b) {
+        const int s0 = s_begin + b * kNormBatch;
         if (s0 >= s_end) break;
-        u32x4_t xa[kGateBatch], ra[kGateBatch], ga[kGateBatch];
+        u32x4_t xa[kNormBatch], ra[kNormBatch], ga[kNormBatch];
 #pragma unroll
-        for (int i = 0; i < kGateBatch; ++i) {
+        for (int i = 0; i < kNormBatch; ++i) {
             const int h = (s0 + i) * 32 + kq * 8;
             const bool okk = (s0 + i < s_end) && (h < H);
             const bool ok = okk && tok_ok;
@@ -172,13 +175,13 @@ __global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
             ga[i] = okk ? *reinterpret_cast<const u32x4_t*>(grow + h) : u32x4_t{0u, 0u, 0u, 0u};
         }
 #pragma unroll
-        for (int i = 0; i < kGateBatch; ++i) {
+        for (int i = 0; i < kNormBatch; ++i) {
             const int h = (s0 + i) * 32 + kq * 8;
             const bool okk = (s0 + i < s_end) && (h < H);
             float sv[8], wv[8];
             if (RESIDENT) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) sv[j] = kept[b * kGateBatch + i][j];
+                for (int j = 0; j < 8; ++j) sv[j] = kept[b * kNormBatch + i][j];
             } else {
                 u32x4_t rounded;
                 row_piece(xa[i], ra[i], sv, rounded);
@@ -220,7 +223,7 @@ __global__ __launch_bounds__(kGateThreads) void norm_gate_router_kernel(
                                                           __builtin_bit_cast(bf16x8_t, yb), acc, 0, 0, 0);
         }
     }
-    reduce_tiles_and_route<E_, kGateWaves>(acc, partial, wave, lane, t0, T, k, renorm, round_bf16, logits_out, out_w,
+    reduce_tiles_and_route<E_, kNormGateWaves>(acc, partial, wave, lane, t0, T, k, renorm, round_bf16, logits_out, out_w,
                                            out_ids);
 }
 
@@ -230,7 +233,7 @@ void launch_norm_gate(bool add, bool layer, unsigned grid, hipStream_t s, const 
                       int renorm, int round_bf16, void* lo, float* w, int32_t* ids) {
     typedef typename WElem::storage WS;
     const WS* nwp = static_cast<const WS*>(nw);
-    const dim3 gd(grid), bd(kGateThreads);
+    const dim3 gd(grid), bd(kNormGateThreads);
     if (add && layer)
         hipLaunchKernelGGL((norm_gate_router_kernel<E_, WElem, true, true, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
     else if (add)
@@ -282,7 +285,7 @@ int launch_norm_gate_router(const void* x_in, const void* res_in, const void* no
     const uint16_t* gp = static_cast<const uint16_t*>(gate_w);
     const bool add = res_in != nullptr;
     const bool w32 = norm_w_dtype == EM_DTYPE_F32;
-    const bool resident = ceil_div(ceil_div(H, 32), kGateWaves) <= kResidentSteps;
+    const bool resident = ceil_div(ceil_div(H, 32), kNormGateWaves) <= kResidentSteps;
 #define EM_NORM_GATE(E_, W_, R_) launch_norm_gate<E_, W_, R_>(add, layer_semantics, grid, s, xp, rp, norm_w, eps, hp, rop, gp, T, H, k, renorm, round_bf16, logits_out, w, ids)
     if (E == 8) {
         if (w32) { if (resident) EM_NORM_GATE(8, F32Elem, true); else EM_NORM_GATE(8, F32Elem, false); }
