@@ -47,6 +47,9 @@ def parse_args():
                     help="values of x and the expert weights.  'zeros' is a diagnostic: the matrix pipes then draw "
                          "little power and the same kernels run at the full shader clock, which separates the "
                          "board's power limit from the kernels' own stalls; never the headline")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="diagnostic: time the library's dense bf16 GEMM of the w13 GEMM's size (torch.matmul, "
+                         "[tokens*top_k, H] x [2I, H]^T) on the same operand distributions, print it and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three device copies of 1 GiB (a plain copy kernel of known size that the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by)")
@@ -195,6 +198,23 @@ def calibrate_copy(torch, dev):
     del src, dst
 
 
+def vendor_gemm(torch, dev, T, steps, warmup):
+    """What the same board does on a dense problem of the w13 GEMM's flops: a yardstick for the power limit."""
+    M, N, K = T * TOPK, 2 * I, H
+    if OPERANDS == "zeros":
+        a = torch.zeros(M, K, device=dev, dtype=torch.bfloat16)
+        b = torch.zeros(N, K, device=dev, dtype=torch.bfloat16)
+    else:
+        g = torch.Generator(device=dev).manual_seed(0)
+        a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+        b = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    c = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+    bt = b.t()
+    ms, _ = time_calls(torch, lambda: torch.matmul(a, bt, out=c), steps, warmup)
+    return {"diagnostic": "library dense bf16 GEMM (torch.matmul)", "M": M, "N": N, "K": K, "operands": OPERANDS,
+            "ms": ms, "tflops": 2.0 * M * N * K / ms / 1e9, "frac_of_peak": 2.0 * M * N * K / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+
+
 def main():
     global H, I, OPERANDS
     args = parse_args()
@@ -217,6 +237,9 @@ def main():
         LayerRunner.base_flags = _lib.FLAG_ACCURATE
     if args.calibrate_copy:
         calibrate_copy(torch, dev)
+    if args.vendor_gemm:
+        print(json.dumps(vendor_gemm(torch, dev, args.tokens, min(args.steps, 30), min(args.warmup, 5))))
+        return
     w13, w2 = make_weights(torch, dev)
 
     T = args.tokens
