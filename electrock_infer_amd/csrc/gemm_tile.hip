@@ -166,6 +166,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             voff[n] = grow * static_cast<uint32_t>(K * 2) + piece * 16;
         }
     }
+    // MODE 2 scatters its rows by slot in the epilogue: fetch the slot of row `tid` now, not at the end of the tile
+    int my_slot = -1;
+    if (MODE == 2 && tid < kTM && tid < valid) my_slot = p.sorted_ids[m0 + tid];
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const int nk = kslice / kTK;
@@ -401,7 +404,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         constexpr int kPitchY = 64 * 4 + 16;
         int32_t* slots = reinterpret_cast<int32_t*>(smem);
         uint8_t* ytile = smem + 1024 + wave * (32 * kPitchY);
-        if (tid < kTM) slots[tid] = (tid < valid) ? p.sorted_ids[m0 + tid] : -1;
+        if (tid < kTM) slots[tid] = my_slot;
         __syncthreads();
         float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
 #pragma unroll
