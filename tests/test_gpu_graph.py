@@ -1,0 +1,66 @@
+"""The layer under HIP graph capture: the library allocates nothing, clears nothing with memset and keeps no
+state between calls, so a captured forward pass must replay to the same bits as the eager one -- also after
+other work has run in between, and with new inputs written into the captured buffers."""
+import pytest
+import torch
+
+from tests.gpu_util import DEV, announce, gpu_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("T,H,I", [(1, 512, 1024), (64, 512, 1024), (300, 512, 1024), (1024, 512, 1024)])
+def test_captured_layer_replays_bit_exact(T, H, I):
+    from electrock_infer_amd.layers.moe.fused_moe import fused_experts, get_workspace
+    announce(f"graph capture T={T}")
+    E = 8
+    x, lg, w13, w2 = gpu_inputs(T, H, I, E, seed=T)
+    ws = get_workspace(x.device, T, H, I, E, 2)
+    eager = fused_experts(x, w13, w2, lg, topk=2, workspace=ws).clone()     # also warms up one-time setup calls
+    static_x, static_lg = x.clone(), lg.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fused_experts(static_x, w13, w2, static_lg, topk=2, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = fused_experts(static_x, w13, w2, static_lg, topk=2, workspace=ws)
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, eager), f"replay {rep}"
+        # eager work of the program between replays, on the same workspace
+        other = fused_experts(x.flip(0).contiguous(), w13, w2, lg.flip(0).contiguous(), topk=2, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(other.flip(0), eager)
+    # new inputs through the captured buffers
+    x2, lg2, _, _ = gpu_inputs(T, H, I, E, seed=T + 1)
+    static_x.copy_(x2)
+    static_lg.copy_(lg2)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(static_out, fused_experts(x2, w13, w2, lg2, topk=2, workspace=ws))
+
+
+def test_captured_decoder_tail_replays_bit_exact():
+    from electrock_infer_amd.layers.moe.fused_moe import fused_experts_normed, get_workspace
+    announce("graph capture, norm + gate + experts")
+    T, H, I, E = 48, 512, 1024, 8
+    x, _, w13, w2 = gpu_inputs(T, H, I, E, seed=5)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    r = torch.randn(T, H, generator=g, device=DEV).to(torch.bfloat16)
+    nw = (1.0 + 0.1 * torch.randn(H, generator=g, device=DEV)).to(torch.bfloat16)
+    gw = (torch.randn(E, H, generator=g, device=DEV) * 0.05).to(torch.bfloat16)
+    ws = get_workspace(x.device, T, H, I, E, 2)
+    out_e, res_e = fused_experts_normed(x, r, nw, 1e-5, gw, w13, w2, topk=2, workspace=ws)
+    out_e, res_e = out_e.clone(), res_e.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, res_g = fused_experts_normed(x, r, nw, 1e-5, gw, w13, w2, topk=2, workspace=ws)
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e) and torch.equal(res_g, res_e), f"replay {rep}"
+        fused_experts_normed(x, r, nw, 1e-5, gw, w13, w2, topk=2, workspace=ws)
+        torch.cuda.synchronize()
