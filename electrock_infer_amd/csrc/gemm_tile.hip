@@ -117,9 +117,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             mt -= t;
         }
     }
-    const int64_t m0 = seg_begin[expert] + static_cast<int64_t>(mt) * kTM;
-    const int rows_left = seg_begin[expert + 1] - static_cast<int>(m0);
-    const int valid = rows_left < kTM ? rows_left : kTM;  // multiple of 32, >= 32
+    // The expert's 32-row blocks are dealt evenly to its row tiles (heights differ by at most one block): every
+    // tile streams the same weight bytes, so a nearly empty last tile would cost a full tile's time.
+    const int e_rows = seg_begin[expert + 1] - seg_begin[expert];
+    const int e_tiles = (e_rows + kTM - 1) / kTM;
+    const int e_blocks = e_rows / kRowBlock;
+    const int blk_base = e_blocks / e_tiles, blk_rem = e_blocks % e_tiles;
+    const int64_t m0 = seg_begin[expert] + static_cast<int64_t>(mt * blk_base + (mt < blk_rem ? mt : blk_rem)) * kRowBlock;
+    const int valid = (blk_base + (mt < blk_rem ? 1 : 0)) * kRowBlock;  // multiple of 32, >= 32
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -223,14 +228,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     // Token fragments live in register set u & 1, weight fragments (shared by both row halves) in set k32.
     bf16x8_t fa[2][4], fb[2][4];
     // operand fragments of unit u of K step stage_k (weight rows in ring slot bslot)
-    auto read_frags = [&](int stage_k, int bslot, int u, auto full_tag) {
-        constexpr bool FULL = decltype(full_tag)::value;
+    // (nmi_tag: the wave's number of 32-row blocks as a constant, 0 = use the runtime value)
+    auto read_frags = [&](int stage_k, int bslot, int u, auto nmi_tag) {
+        constexpr int NMI = decltype(nmi_tag)::value;
         const int h = u & 1, k32 = u >> 1;
         const uint8_t* sa = smem + (stage_k & 1) * kSlotBytes;
         const uint8_t* sb = smem + bslot * kSlotBytes;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if (FULL || h * 4 + j < 2 * nmi)
+            if (NMI ? (h * 4 + j < 2 * NMI) : (h * 4 + j < 2 * nmi))
                 fa[h][j] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[k32] + (h * 4 + j) * 2048);
         if (h == 0) {
 #pragma unroll
@@ -238,13 +244,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         }
     };
     // the 16 MFMAs of unit u; `reads` LDS reads issued just before the call are spread one behind each of the first MFMAs
-    auto multiply = [&](int u, auto reads_tag, auto full_tag) {
-        constexpr bool FULL = decltype(full_tag)::value;
+    auto multiply = [&](int u, auto reads_tag, auto nmi_tag) {
+        constexpr int NMI = decltype(nmi_tag)::value;
+        constexpr bool FULL = NMI == 4;
         constexpr int reads = decltype(reads_tag)::value;
         const int h = u & 1, k32 = u >> 1;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if (FULL || h * 4 + j < 2 * nmi) {
+            if (NMI ? (h * 4 + j < 2 * NMI) : (h * 4 + j < 2 * nmi)) {
 #pragma unroll
                 for (int gi = 0; gi < 4; ++gi) {
                     const int g = (j & 1) ? 3 - gi : gi;  // serpentine: one operand changes between neighbours
@@ -280,17 +287,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     if (1 < nk) issue_a(1);
     if (2 < nk) issue_b(2, 2);
     int bs = 0;  // ring slot of the weight rows of step kt
-    if (nmi == 4) {
-        // All four fragments exist (the common case): fixed instruction mix.  After the barrier that ends step
-        // kt, the eight MFMAs of its last 16-wide K step alternate with the copies of A(kt+2) and B(kt+3) (the
-        // slots step kt has just freed) and with the first operand reads of step kt+1.
-        const std::true_type full;
-        read_frags(0, 0, 0, full);
+    // The main loop for a wave with NMI = 1 .. 4 blocks of 32 rows (a compile-time constant: fixed instruction
+    // mix).  After the barrier that ends step kt, the MFMAs of its last unit alternate with the copies of A(kt+2)
+    // and B(kt+3) (the slots step kt has just freed) and with the first operand reads of step kt+1.
+    auto main_loop = [&](auto nmi_tag) {
+        constexpr int NMI = decltype(nmi_tag)::value;
+        read_frags(0, 0, 0, nmi_tag);
         auto step = [&](int kt, auto copy_a_tag, auto copy_b_tag) {
             constexpr bool CA = decltype(copy_a_tag)::value, CB = decltype(copy_b_tag)::value;
-            read_frags(kt, bs, 1, full); multiply(0, r4, full);
-            read_frags(kt, bs, 2, full); multiply(1, r8, full);
-            read_frags(kt, bs, 3, full); multiply(2, r4, full);
+            read_frags(kt, bs, 1, nmi_tag); multiply(0, r4, nmi_tag);
+            read_frags(kt, bs, 2, nmi_tag); multiply(1, r8, nmi_tag);
+            read_frags(kt, bs, 3, nmi_tag); multiply(2, r4, nmi_tag);
             if (CA) wait_dma<kDmaHalf>(); else wait_dma<0>();   // this wave's parts of A(kt+1), B(kt+1) are in LDS
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of step kt are in registers
             block_barrier();                                    // ... and so are everyone else's
@@ -299,21 +306,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             const uint8_t* sa = smem + ((kt + 1) & 1) * kSlotBytes;
             const uint8_t* sb = smem + bn * kSlotBytes;
             // unit 3 of step kt; behind every second MFMA a copy, behind the others a read of unit 0 of step kt+1
-            // (weight fragment 0 and token fragment 0 first: the next unit starts with them)
+            // (weight fragment 0 and token fragment 0 first: the next unit starts with them).  A wave with fewer
+            // than four blocks has fewer (or no) MFMAs here; its copies and reads keep their places.
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int j = i >> 2, g = (j & 1) ? 3 - (i & 3) : (i & 3);  // serpentine, as in multiply()
-                acc[4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][j], fb[1][g], acc[4 + j][g], 0, 0, 0);
+                if (4 + j < 2 * NMI)
+                    acc[4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][j], fb[1][g], acc[4 + j][g], 0, 0, 0);
                 const int n = i >> 1;
                 if ((i & 1) == 0) {
-                    if (n < 4) { if (CA) copy_a(n, kt + 2); } else { if (CB) copy_b(n - 4, kt + 3, bs); }
+                    if (n < 4) { if (CA && (NMI == 4 || live[n])) copy_a(n, kt + 2); } else { if (CB) copy_b(n - 4, kt + 3, bs); }
                 } else if (n == 0) {
                     fb[0][0] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0]);
                 } else if (n == 1) {
                     fa[0][0] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0]);
                 } else if (n < 5) {
                     fb[0][n - 1] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0] + (n - 1) * 2048);
-                } else {
+                } else if (n - 4 < 2 * NMI) {
                     fa[0][n - 4] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0] + (n - 4) * 2048);
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -324,14 +333,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         for (; kt + 3 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
         for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::false_type{});
         for (; kt + 1 < nk; ++kt) step(kt, std::false_type{}, std::false_type{});
-        read_frags(nk - 1, bs, 1, full); multiply(0, r4, full);
-        read_frags(nk - 1, bs, 2, full); multiply(1, r8, full);
-        read_frags(nk - 1, bs, 3, full); multiply(2, r4, full);
-        multiply(3, r0, full);
+        read_frags(nk - 1, bs, 1, nmi_tag); multiply(0, r4, nmi_tag);
+        read_frags(nk - 1, bs, 2, nmi_tag); multiply(1, r8, nmi_tag);
+        read_frags(nk - 1, bs, 3, nmi_tag); multiply(2, r4, nmi_tag);
+        multiply(3, r0, nmi_tag);
+    };
+    if (nmi == 4) {
+        main_loop(std::integral_constant<int, 4>{});
+    } else if (nmi == 3) {
+        main_loop(std::integral_constant<int, 3>{});
+    } else if (nmi == 2) {
+        main_loop(std::integral_constant<int, 2>{});
+    } else if (nmi == 1) {
+        main_loop(std::integral_constant<int, 1>{});
     } else {
-        // Short tile: a wave multiplies the fragments that exist; waves without rows still copy and meet the
-        // barriers.  Skipped copies of missing token rows do not change the counts: the newest four are B's.
-        const std::false_type part;
+        // A wave without rows (the tile is at most 128 rows high) still copies and meets the barriers.
+        // Skipped copies of missing token rows do not change the counts: the newest four are B's.
+        const std::integral_constant<int, 0> part;
         const bool work = nmi > 0;
         if (work) read_frags(0, 0, 0, part);
         for (int kt = 0; kt + 1 < nk; ++kt) {
