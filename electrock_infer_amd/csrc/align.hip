@@ -81,10 +81,16 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
     __syncthreads();  // also orders the -1 / 0 fill before the scatter below
     if (seg_out != nullptr && tid <= E) seg_out[tid] = seg_begin[tid];  // padded start of every expert segment
 
-    // block -> expert table
-    if (tid < E) {
-        for (int32_t p = seg_begin[tid]; p < seg_begin[tid + 1]; p += block)
-            if (p / block < eid_len) expert_ids[p / block] = tid;
+    // block -> expert table: every thread looks its blocks up in the segment starts (a hot expert has
+    // thousands of blocks: one thread per expert would walk them alone)
+    {
+        const int64_t nblocks = seg_begin[E] / block;
+        for (int64_t b = tid; b < nblocks && b < eid_len; b += kAlignThreads) {
+            const int32_t row = static_cast<int32_t>(b) * block;
+            int e = 0;
+            while (e + 1 < E && row >= seg_begin[e + 1]) ++e;
+            expert_ids[b] = e;
+        }
     }
 
     // ---- pass 2: stable scatter ----
