@@ -22,14 +22,16 @@ namespace {
 constexpr int kAlignThreads = 1024;
 constexpr int kAlignWaves = kAlignThreads / kWave;
 
-template <typename IdT>
+// EC: the number of experts as a compile-time constant (the ballot loops unroll), 0 = use the argument
+template <typename IdT, int EC>
 __global__ __launch_bounds__(kAlignThreads) void align_kernel(
-    const IdT* __restrict__ ids, int64_t numel, int E, int block,
+    const IdT* __restrict__ ids, int64_t numel, int E_arg, int block,
     int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
     int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out) {
     __shared__ int32_t hist[kAlignWaves][kMaxExperts];  // pass 1 counts, then write bases
     __shared__ int32_t seg_begin[kMaxExperts + 1];      // padded exclusive prefix
 
+    const int E = EC ? EC : E_arg;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -48,9 +50,15 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
     for (int64_t i0 = begin; i0 < end; i0 += kWave) {
         const int64_t i = i0 + lane;
         const int e = (i < end) ? static_cast<int>(ids[i]) : -1;
-        for (int j = 0; j < E; ++j) {
+        auto count_expert = [&](int j) {
             const uint64_t m = __ballot(e == j);
             if (lane == j) cnt += __popcll(m);
+        };
+        if (EC) {
+#pragma unroll
+            for (int j = 0; j < EC; ++j) count_expert(j);
+        } else {
+            for (int j = 0; j < E; ++j) count_expert(j);
         }
     }
     if (lane < kMaxExperts) hist[wave][lane] = (lane < E) ? cnt : 0;
@@ -101,10 +109,16 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
         const bool valid = (e >= 0 && e < E);
         const int32_t base = __shfl(pos, valid ? e : 0);
         int32_t rank = 0;
-        for (int j = 0; j < E; ++j) {
+        auto rank_expert = [&](int j) {
             const uint64_t m = __ballot(e == j);
             if (e == j) rank = __popcll(m & lt_mask);
             if (lane == j) pos += __popcll(m);
+        };
+        if (EC) {
+#pragma unroll
+            for (int j = 0; j < EC; ++j) rank_expert(j);
+        } else {
+            for (int j = 0; j < E; ++j) rank_expert(j);
         }
         if (valid && base + rank < sorted_len) sorted[base + rank] = static_cast<int32_t>(i);
     }
@@ -117,10 +131,14 @@ int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* post_pad, int32_t* seg_out, hipStream_t s) {
     const dim3 grid(1), blk(kAlignThreads);
     if (itype == EM_ITYPE_I32) {
-        hipLaunchKernelGGL(align_kernel<int32_t>, grid, blk, 0, s, static_cast<const int32_t*>(ids),
-                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
+        if (E == 8)
+            hipLaunchKernelGGL((align_kernel<int32_t, 8>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
+                               numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
+        else
+            hipLaunchKernelGGL((align_kernel<int32_t, 0>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
+                               numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else if (itype == EM_ITYPE_I64) {
-        hipLaunchKernelGGL(align_kernel<int64_t>, grid, blk, 0, s, static_cast<const int64_t*>(ids),
+        hipLaunchKernelGGL((align_kernel<int64_t, 0>), grid, blk, 0, s, static_cast<const int64_t*>(ids),
                            numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else {
         return EM_ERR_BAD_DTYPE;
