@@ -197,8 +197,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
         for (int j = 0; j < top_k; ++j) {
             const float wj = w[t * top_k + j];
             const float* row = y + (t * top_k + j) * static_cast<int64_t>(H) + h;
-            f32x4_t s = *reinterpret_cast<const f32x4_t*>(row);
-            for (int z = 1; z < ksplit; ++z) s += *reinterpret_cast<const f32x4_t*>(row + z * zstride);
+            // the partial results are read exactly once: streaming loads
+            f32x4_t s = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(row));
+            for (int z = 1; z < ksplit; ++z) s += __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(row + z * zstride));
             acc += wj * s;
         }
         if (kOutF32) {
