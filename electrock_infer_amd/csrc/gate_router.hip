@@ -73,6 +73,7 @@ __global__ __launch_bounds__(kGateThreads) void gate_router_kernel(
 constexpr int kNormGateWaves = 16;   // 1024 threads: 64 kept values per lane leave room for four waves per SIMD
 constexpr int kNormGateThreads = kNormGateWaves * kWave;
 constexpr int kNormBatch = 4;        // K steps whose loads are in flight together (8 would spill)
+constexpr int64_t kFusedNormMaxT = 16;  // up to here norm + gate + router share one launch
 constexpr int kResidentSteps = 8;    // K steps of 32 a wave keeps in registers: 16 waves x 8 x 32 = 4096
 template <int E_, typename WElem, bool ADD, bool LAYER, bool RESIDENT>
 __global__ __launch_bounds__(kNormGateThreads) void norm_gate_router_kernel(
@@ -277,6 +278,15 @@ int launch_norm_gate_router(const void* x_in, const void* res_in, const void* no
     if (T == 0) return 0;
     if (!gate_router_supported(H, E)) return EM_ERR_UNSUPPORTED;
     if (norm_w_dtype != EM_DTYPE_BF16 && norm_w_dtype != EM_DTYPE_F32) return EM_ERR_BAD_DTYPE;
+    // One launch pays while the launch itself is what costs (a single workgroup: 14 against 9 + 9 us at T = 1).
+    // Beyond that the row-per-workgroup norm kernel followed by the gate kernel is as fast or faster (the fused
+    // workgroup is a chain of load, reduce, barrier, scale and store, with one workgroup per CU), so those run.
+    if (T > kFusedNormMaxT && rms_norm_supported(H, EM_DTYPE_BF16, norm_w_dtype)) {
+        const int rc = launch_rms_norm(x_in, res_in, norm_w, h_out, res_out, T, H, eps, EM_DTYPE_BF16, norm_w_dtype,
+                                       layer_semantics, s);
+        if (rc != 0) return rc;
+        return launch_gate_router(h_out, gate_w, T, H, E, k, renorm, round_bf16, logits_out, w, ids, s);
+    }
     const unsigned grid = static_cast<unsigned>(ceil_div(T, static_cast<int64_t>(kGateTokens)));
     const uint16_t* xp = static_cast<const uint16_t*>(x_in);
     const uint16_t* rp = static_cast<const uint16_t*>(res_in);
