@@ -186,7 +186,9 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(MoeProblem p) {
 }
 
 // out[t, :] = sum_j w[t, j] * sum_z y[z, t*k + j, :]   (fp32, one final rounding)
-template <bool kOutF32>
+// kStream: the partial results are too many to still sit in the caches when they are read (exactly once):
+// streaming loads.  Small sets are read back out of L2, where streaming loads of just-written lines are slower.
+template <bool kOutF32, bool kStream>
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
                                                       void* __restrict__ out, int64_t T, int H, int top_k,
                                                       int ksplit) {
@@ -197,9 +199,12 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
         for (int j = 0; j < top_k; ++j) {
             const float wj = w[t * top_k + j];
             const float* row = y + (t * top_k + j) * static_cast<int64_t>(H) + h;
-            // the partial results are read exactly once: streaming loads
-            f32x4_t s = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(row));
-            for (int z = 1; z < ksplit; ++z) s += __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(row + z * zstride));
+            auto load = [](const float* ptr) {
+                return kStream ? __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(ptr))
+                               : *reinterpret_cast<const f32x4_t*>(ptr);
+            };
+            f32x4_t s = load(row);
+            for (int z = 1; z < ksplit; ++z) s += load(row + z * zstride);
             acc += wj * s;
         }
         if (kOutF32) {
@@ -239,12 +244,13 @@ int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
     if (p.T == 0) return 0;
     const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 1024));
     const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
-    if (out_f32)
-        hipLaunchKernelGGL(combine_kernel<true>, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k,
-                           p.ksplit);
-    else
-        hipLaunchKernelGGL(combine_kernel<false>, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k,
-                           p.ksplit);
+    // beyond the memory-side cache (256 MB) the partial results come back from HBM
+    const bool stream = static_cast<int64_t>(p.ksplit) * p.T * p.top_k * p.H * 4 > (int64_t{256} << 20);
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k, p.ksplit);
+    };
+    if (out_f32) { if (stream) go(combine_kernel<true, true>); else go(combine_kernel<true, false>); }
+    else { if (stream) go(combine_kernel<false, true>); else go(combine_kernel<false, false>); }
     return launch_status();
 }
 
