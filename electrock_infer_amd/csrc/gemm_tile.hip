@@ -4,12 +4,15 @@
 //   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile of up to 256 sorted rows x 256
 //              weight rows; K in steps of 64; LDS (all 160 KB) holds a ring of two 32 KB
 //              slots of token rows (A) and a ring of three 32 KB slots of weight rows (B)
-//   tiles      the sort pads experts to 32 rows only; every expert is cut into 256-row
-//              tiles and its last tile is as high as the rows that are left (a multiple
-//              of 32).  A wave multiplies only the 32-row fragments that exist, so a
-//              short tile costs its share of MFMA time, and its missing A rows are not
-//              fetched.  The tile list is rebuilt by every workgroup from the per-expert
-//              segment starts (at most 64 scalar loads).
+//   tiles      the sort pads experts to 32 rows only; an expert with r rows gets ceil(r / 256)
+//              row tiles and its 32-row blocks are dealt evenly to them (heights differ by
+//              one block at most): every tile streams the same weight bytes whatever its
+//              height, so a full-height tiling with a nearly empty last tile cost a full
+//              tile's time for a few rows, and equal tiles stay in step and share through
+//              L2.  A wave multiplies only the blocks it has -- its main loop is instantiated
+//              for 1 .. 4 blocks -- and missing A rows are not fetched.  The tile list is
+//              rebuilt by every workgroup from the per-expert segment starts (at most 64
+//              scalar loads).
 //   loads      global -> LDS directly (global_load_lds_dwordx4), no registers in
 //              between; eight lanes fetch one full 128-byte line of a row (measured
 //              L2 -> CU feed: ~26 TB/s with 128 B per row against ~17 TB/s with 64 B).
@@ -19,7 +22,7 @@
 //              on the critical path of every step.  Completion is tracked by hand with
 //              s_waitcnt vmcnt + one s_barrier per step.
 //   issue      the eight copy instructions of a wave are issued one by one between the
-//              eight MFMAs that follow the barrier: issued back to back (by both waves of
+//              MFMAs that follow the barrier: issued back to back (by both waves of
 //              a SIMD at once) they left the matrix pipe idle for a fifth of every step
 //   LDS        rows are 128 B; the 16-byte pieces of every 2-row group are XOR-
 //              swizzled so that the 16 lanes of a b128 operand read hit 16 bank groups
