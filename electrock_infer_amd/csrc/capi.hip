@@ -15,6 +15,10 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 // Up to this many tokens the weight-streaming GEMM runs (16-row sorted blocks, a
 // couple of MFMA fragments per expert); above it the tiled kernels take over.
 constexpr int64_t kStreamMaxT = 64;
+// Above this many tokens the w2 GEMM of a streaming-size batch runs on the 64-row tiled kernel (same sorted
+// layout): it holds its speed when experts get a second MFMA fragment of rows, where the streaming kernel loses
+// 10 % (8x7B) and is 20 % ahead throughout on the 8x22B shape.
+constexpr int64_t kStreamW2MaxT = 16;
 // Tile height of the tiled kernels by batch size (8 experts, top-2: T/4 rows per expert on
 // average): 64-row tiles while most experts fit one of them, 128-row tiles likewise, then the
 // 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 448 tokens.
@@ -39,10 +43,11 @@ inline int choose_ksplit(int64_t T, int H, int I) {
         return 1;
     }
     // Streaming kernel: (active experts) x (H / 64) row tiles should give every CU
-    // work.  From ~17 tokens on all eight experts are almost surely active and one
-    // K slice per tile measures fastest; below that the reduction is split four ways.
-    // The kernel needs I / ksplit to be a multiple of 256.
-    const int want = T <= 16 ? 4 : 1;
+    // work; up to 16 tokens the reduction is split four ways.  Above that the 64-row tiled
+    // kernel takes the w2 GEMM with two K slices where the shape allows it, else the streaming
+    // kernel with one.  The streaming kernel needs I / ksplit to be a multiple of 256, which
+    // covers the tiled kernel's 64.
+    const int want = T <= kStreamW2MaxT ? 4 : (tile_shape_ok(H, I) ? 2 : 1);
     for (int ks = want; ks >= 1; --ks)
         if (I % (ks * 256) == 0) return ks;
     return want;
@@ -268,7 +273,9 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
-        if (use_stream) {
+        if (use_stream && !accurate && T > kStreamW2MaxT && p.ksplit >= 2 && tile_mid_supported(p)) {
+            rc = launch_gemm_tile_mid(p, seg_begin, 2, 64, s);
+        } else if (use_stream) {
             rc = launch_gemm_stream(p, seg_begin, 2, s);  // multiplies act and act_lo in one pass
         } else {
             rc = use_tile ? tile_gemm(p, 2) : launch_gemm_generic(p, 2, s);

@@ -268,6 +268,17 @@ def test_layer_mid_shape_all_tile_cases(T, routing):
     check_outputs(f"mid_T{T}_{routing}_generic", gen_f32.cpu(), gen_bf16.cpu(), ref)
 
 
+@pytest.mark.parametrize("T", [96, 300])
+def test_layer_mid_kernel_wide_w13_tiles(T):
+    """I = 4096 makes 8 experts x 32 column tiles = one full round of CUs, so the w13 GEMM of the 64- and
+    128-row kernels keeps its 256-row weight tiles (the other shapes in this file get the 128-row ones)."""
+    announce(f"layer H=256 I=4096 T={T}")
+    x, lg, w13, w2 = O.make_inputs(T, 256, 4096, seed=T)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    out_f32, out_bf16 = run_both(*(t.to(DEV) for t in (x, lg, w13, w2)))
+    check_outputs(f"wide_T{T}", out_f32.cpu(), out_bf16.cpu(), ref)
+
+
 @pytest.mark.parametrize("T", [1, 7, 33, 64])
 @pytest.mark.parametrize("routing", ["normal", "two_experts", "one_expert"])
 def test_layer_mid_shape_decode_cases(T, routing):
