@@ -15,6 +15,7 @@
 // (layers/moe/moe_align_block_size.py:32-48): pads and tail of sorted ids are -1,
 // unused tail of expert_ids is 0.
 #include "common.h"
+#include "router_device.h"
 
 namespace em {
 namespace {
@@ -22,14 +23,15 @@ namespace {
 constexpr int kAlignThreads = 1024;
 constexpr int kAlignWaves = kAlignThreads / kWave;
 
+// The sort, run by one workgroup of kAlignThreads threads; `ids` may live in global memory or in LDS.
+// hist: pass 1 counts, then write bases; seg_begin: padded exclusive prefix (both in LDS).
 // EC: the number of experts as a compile-time constant (the ballot loops unroll), 0 = use the argument
 template <typename IdT, int EC>
-__global__ __launch_bounds__(kAlignThreads) void align_kernel(
+__device__ __forceinline__ void align_body(
     const IdT* __restrict__ ids, int64_t numel, int E_arg, int block,
     int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
-    int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out) {
-    __shared__ int32_t hist[kAlignWaves][kMaxExperts];  // pass 1 counts, then write bases
-    __shared__ int32_t seg_begin[kMaxExperts + 1];      // padded exclusive prefix
+    int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out,
+    int32_t (*hist)[kMaxExperts], int32_t* seg_begin) {
 
     const int E = EC ? EC : E_arg;
     const int tid = threadIdx.x;
@@ -124,6 +126,51 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
     }
 }
 
+template <typename IdT, int EC>
+__global__ __launch_bounds__(kAlignThreads) void align_kernel(
+    const IdT* __restrict__ ids, int64_t numel, int E_arg, int block,
+    int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
+    int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out) {
+    __shared__ int32_t hist[kAlignWaves][kMaxExperts];
+    __shared__ int32_t seg_begin[kMaxExperts + 1];
+    align_body<IdT, EC>(ids, numel, E_arg, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out, hist,
+                        seg_begin);
+}
+
+// Router and sort in one launch for batches whose k * T selected experts fit LDS (the layer then starts its
+// GEMMs one kernel launch earlier: a few microseconds of a decode step).  Eight experts: eight lanes per token
+// as in the stand-alone router; the selected ids go to LDS, from there to topk_ids and into the sort.
+constexpr int kFusedMaxSlots = 4096;
+template <typename Elem>
+__global__ __launch_bounds__(kAlignThreads) void route_align_kernel(
+    const typename Elem::storage* __restrict__ logits, int64_t T, int k, int renorm, float* __restrict__ out_w,
+    int32_t* __restrict__ out_ids, int block, int32_t* __restrict__ sorted, int64_t sorted_len,
+    int32_t* __restrict__ expert_ids, int64_t eid_len, int32_t* __restrict__ post_pad,
+    int32_t* __restrict__ seg_out) {
+    constexpr int E = 8, G = 8, kTokens = kWave / G;
+    __shared__ int32_t hist[kAlignWaves][kMaxExperts];
+    __shared__ int32_t seg_begin[kMaxExperts + 1];
+    __shared__ int32_t ids[kFusedMaxSlots];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    for (int64_t t0 = 0; t0 < T; t0 += kAlignWaves * kTokens) {  // same trip count for every wave
+        const int64_t t = t0 + wave * kTokens + lane / G;
+        const bool valid = t < T;
+        float v = -INFINITY;
+        if (valid) {
+            v = Elem::load(logits[t * E + (lane & (G - 1))]);
+            if (v != v) v = -INFINITY;  // a NaN logit can never be selected
+        }
+        route_group<G>(v, lane, t, valid, E, k, renorm, out_w, ids);
+    }
+    __syncthreads();
+    const int64_t numel = T * k;
+    for (int64_t i = tid; i < numel; i += kAlignThreads) out_ids[i] = ids[i];
+    align_body<int32_t, E>(ids, numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out, hist,
+                           seg_begin);
+}
+
 }  // namespace
 
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
@@ -142,6 +189,25 @@ int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                            numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else {
         return EM_ERR_BAD_DTYPE;
+    }
+    return launch_status();
+}
+
+bool route_align_supported(int64_t T, int E, int k) { return E == 8 && T > 0 && T * k <= kFusedMaxSlots; }
+
+int launch_route_align(const void* logits, int logits_dtype, int64_t T, int k, int renorm, float* w, int32_t* ids,
+                       int block, int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
+                       int32_t* post_pad, int32_t* seg_out, hipStream_t s) {
+    const dim3 grid(1), blk(kAlignThreads);
+    auto go = [&](auto kernel, auto* lp) {
+        hipLaunchKernelGGL(kernel, grid, blk, 0, s, lp, T, k, renorm, w, ids, block, sorted, sorted_len, expert_ids,
+                           eid_len, post_pad, seg_out);
+    };
+    switch (logits_dtype) {
+        case EM_DTYPE_F32: go(route_align_kernel<F32Elem>, static_cast<const F32Elem::storage*>(logits)); break;
+        case EM_DTYPE_BF16: go(route_align_kernel<BF16Elem>, static_cast<const BF16Elem::storage*>(logits)); break;
+        case EM_DTYPE_F16: go(route_align_kernel<F16Elem>, static_cast<const F16Elem::storage*>(logits)); break;
+        default: return EM_ERR_BAD_DTYPE;
     }
     return launch_status();
 }

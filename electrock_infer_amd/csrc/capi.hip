@@ -243,7 +243,14 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.sorted_len = L.sorted_len;
     p.ksplit = static_cast<int>(L.ksplit);
 
-    if (!(flags & EM_FLAG_SKIP_ROUTER)) {
+    const bool fused_front = !(flags & (EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN)) && norm == nullptr &&
+                             gate_w == nullptr && route_align_supported(T, E, top_k);
+    if (fused_front) {
+        rc = launch_route_align(router_logits, logits_dtype, T, top_k, renormalize, topk_w, topk_ids, p.block, sorted,
+                                L.sorted_len, eids, L.expert_ids_len, post_pad, seg_begin, s);
+        if (rc != 0) return rc;
+    }
+    if (!fused_front && !(flags & EM_FLAG_SKIP_ROUTER)) {
         const int round_logits = (flags & EM_FLAG_GATE_F32_LOGITS) ? 0 : 1;
         if (norm != nullptr)
             rc = launch_norm_gate_router(norm->x_in, norm->residual_in, norm->weight, norm->weight_dtype, norm->eps,
@@ -255,7 +262,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
             rc = launch_router(router_logits, logits_dtype, T, E, top_k, renormalize, topk_w, topk_ids, s);
         if (rc != 0) return rc;
     }
-    if (!(flags & EM_FLAG_SKIP_ALIGN)) {
+    if (!fused_front && !(flags & EM_FLAG_SKIP_ALIGN)) {
         rc = launch_align(topk_ids, EM_ITYPE_I32, T * top_k, E, p.block, sorted, L.sorted_len, eids,
                           L.expert_ids_len, post_pad, seg_begin, s);
         if (rc != 0) return rc;

@@ -94,6 +94,11 @@ int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
                  int32_t* post_pad, int32_t* seg_out /* [E+1] padded segment starts, may be null */,
                  hipStream_t s);
+// Router + sort in one launch (eight experts, k * T slots within the kernel's LDS table).
+bool route_align_supported(int64_t T, int E, int k);
+int launch_route_align(const void* logits, int logits_dtype, int64_t T, int k, int renorm, float* w, int32_t* ids,
+                       int block, int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
+                       int32_t* post_pad, int32_t* seg_out, hipStream_t s);
 int launch_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, hipStream_t s);
 int launch_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype, hipStream_t s);
 bool rms_norm_supported(int H, int dtype, int weight_dtype);

@@ -268,6 +268,22 @@ def test_layer_mid_shape_all_tile_cases(T, routing):
     check_outputs(f"mid_T{T}_{routing}_generic", gen_f32.cpu(), gen_bf16.cpu(), ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T", [1, 129, 2048, 2049])
+def test_layer_router_and_sort_in_one_launch(T, dtype):
+    """Up to 2048 tokens (4096 selected experts) the layer routes and sorts in one kernel, above in two: both
+    leave the oracle's routing in the workspace, for every logits type, rows of ties included."""
+    announce(f"layer routing front T={T} logits {dtype}")
+    x, lg, w13, w2 = O.make_inputs(T, 256, 512, seed=T)
+    lg = lg.float()
+    lg[::7] = lg[::7].round()                      # rows with many ties
+    lg[::11, 3] = 60000.0                          # one expert far ahead (finite in every logits type)
+    lg = lg.to(dtype)
+    out = fused_experts(x.to(DEV), w13.to(DEV), w2.to(DEV), lg.to(DEV), 2, out_dtype=torch.float32)
+    assert out.shape == (T, 256)
+    check_routing(get_workspace(DEV, T, 256, 512, 8, 2), lg.float(), T)
+
+
 @pytest.mark.parametrize("T", [96, 300])
 def test_layer_mid_kernel_wide_w13_tiles(T):
     """I = 4096 makes 8 experts x 32 column tiles = one full round of CUs, so the w13 GEMM of the 64- and
