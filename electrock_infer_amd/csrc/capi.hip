@@ -17,8 +17,9 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 constexpr int64_t kStreamMaxT = 64;
 // Above this many tokens the w2 GEMM of a streaming-size batch runs on the 64-row tiled kernel (same sorted
 // layout): it holds its speed when experts get a second MFMA fragment of rows, where the streaming kernel loses
-// 10 % (8x7B) and is 20 % ahead throughout on the 8x22B shape.
-constexpr int64_t kStreamW2MaxT = 16;
+// 10 % (8x7B; T=16: 138 against 146 us, T=12: 121 against 126, T=8: equal, T=5: 98 against 90) and is 20 % ahead
+// throughout on the 8x22B shape.
+constexpr int64_t kStreamW2MaxT = 8;
 // Tile height of the tiled kernels by batch size (8 experts, top-2: T/4 rows per expert on
 // average): 64-row tiles while most experts fit one of them, 128-row tiles likewise, then the
 // 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 448 tokens.
@@ -43,7 +44,7 @@ inline int choose_ksplit(int64_t T, int H, int I) {
         return 1;
     }
     // Streaming kernel: (active experts) x (H / 64) row tiles should give every CU
-    // work; up to 16 tokens the reduction is split four ways.  Above that the 64-row tiled
+    // work; up to 8 tokens the reduction is split four ways.  Above that the 64-row tiled
     // kernel takes the w2 GEMM with two K slices where the shape allows it, else the streaming
     // kernel with one.  The streaming kernel needs I / ksplit to be a multiple of 256, which
     // covers the tiled kernel's 64.
