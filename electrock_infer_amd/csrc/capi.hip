@@ -22,9 +22,9 @@ constexpr int64_t kStreamMaxT = 64;
 constexpr int64_t kStreamW2MaxT = 8;
 // Tile height of the tiled kernels by batch size (8 experts, top-2: T/4 rows per expert on
 // average): 64-row tiles while most experts fit one of them, 128-row tiles likewise, then the
-// 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 448 tokens.
+// 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 352 tokens.
 constexpr int64_t kTile64MaxT = 192;
-constexpr int64_t kTile128MaxT = 448;
+constexpr int64_t kTile128MaxT = 352;
 
 // Rows per sorted block, the counterpart of _get_moe_config (fused_moe.py:327-339):
 // 16 (one MFMA fragment) for the streaming kernel, 32 for the tiled kernel, which cuts

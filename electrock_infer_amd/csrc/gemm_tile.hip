@@ -180,17 +180,29 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const int nk = kslice / kTK;
+    // While every weight byte is read by one workgroup only (STREAM) the w13 tiles start at different K offsets and
+    // wrap around, as in the 64- / 128-row kernel: tiles in step ask for the same 128 bytes of all their rows at once
+    // and load the memory channels unevenly (T=512: 401 -> 353 us, T=768: 433 -> 416 us).  Larger batches keep the
+    // tiles of an XCD in step, they share token rows and weights through L2; the w2 tiles share act rows at every size.
+    // The offset depends on expert and column tile only, so a row's sum keeps one order whatever batch it comes in.
+    constexpr bool kRotate = STREAM && MODE == 1;
+    const int rot = kRotate ? __builtin_amdgcn_readfirstlane((nt * 9 + expert * 3) % nk) : 0;
+    auto krot = [&](int stage_k) {
+        if (!kRotate) return stage_k;
+        const int k = stage_k + rot;
+        return __builtin_amdgcn_readfirstlane(k >= nk ? k - nk : k);
+    };
     // copy n (0..3) of the token rows / weight rows of K step stage_k
     auto copy_a = [&](int n, int stage_k) {
-        dma16(voff[n], base_a + static_cast<int64_t>(stage_k) * (kTK * 2),
+        dma16(voff[n], base_a + static_cast<int64_t>(krot(stage_k)) * (kTK * 2),
               dma_base + (stage_k & 1) * kSlotBytes + n * 8192);
     };
     auto copy_b = [&](int n, int stage_k, int slot) {
         if (STREAM)
-            dma16_stream(voff[kDmaHalf + n], base_b + static_cast<int64_t>(stage_k) * (kTK * 2),
+            dma16_stream(voff[kDmaHalf + n], base_b + static_cast<int64_t>(krot(stage_k)) * (kTK * 2),
                          dma_base + kOffB + slot * kSlotBytes + n * 8192);
         else
-            dma16(voff[kDmaHalf + n], base_b + static_cast<int64_t>(stage_k) * (kTK * 2),
+            dma16(voff[kDmaHalf + n], base_b + static_cast<int64_t>(krot(stage_k)) * (kTK * 2),
                   dma_base + kOffB + slot * kSlotBytes + n * 8192);
     };
     auto issue_a = [&](int stage_k) {
