@@ -14,7 +14,8 @@ One JSON line is printed.  Besides the contract fields it carries
   cpu_baseline  the reference-style torch CPU expert loop (oracle port) timed on
                 the host cores on the same workload
   table         layer latency / HBM GB/s / MFMA TFLOP/s for the other batch sizes
-                of the decode list and the T=8192 prefill case
+                of the decode list, the headline batch in accurate mode and the
+                T=8192 prefill cases
 """
 import argparse
 import json
@@ -42,7 +43,8 @@ def parse_args():
     ap.add_argument("--shape", choices=["8x7b", "8x22b"], default="8x7b",
                     help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
     ap.add_argument("--accurate", action="store_true",
-                    help="run the layer with EM_FLAG_ACCURATE (bf16 hi+lo activations through the w2 GEMM)")
+                    help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 or as a bf16 value + residual "
+                         "pair through the w2 GEMM instead of one bf16)")
     ap.add_argument("--operands", choices=["gaussian", "zeros"], default="gaussian",
                     help="values of x and the expert weights.  'zeros' is a diagnostic: the matrix pipes then draw "
                          "little power and the same kernels run at the full shader clock, which separates the "
@@ -264,6 +266,13 @@ def main():
         for t in ((1, 8, 32, 64, 256) if args.shape == "8x7b" else (1, 64)):
             if t != T:
                 table.append(measure(torch, t, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2)))
+        if not args.accurate:  # the headline batch in accurate mode (activations kept beyond bf16)
+            from electrock_infer_amd import _lib
+            LayerRunner.base_flags = _lib.FLAG_ACCURATE
+            r = measure(torch, T, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2))
+            LayerRunner.base_flags = 0
+            r["accurate_mode"] = True
+            table.append(r)
         for lgk in (("normal", "zipf", "two_experts") if args.shape == "8x7b" else ("normal",)):
             r = measure(torch, 8192 if args.shape == "8x7b" else 4096, w13, w2, 10, 3, logits=lgk)
             r["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS

@@ -223,6 +223,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.act = reinterpret_cast<uint16_t*>(ws + L.act_off);
     const bool accurate = (flags & EM_FLAG_ACCURATE) != 0;
     p.act_lo = accurate ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
+    p.act_f16 = 0;
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
@@ -270,6 +271,16 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     }
     const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
     const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T > kStreamMaxT && tile_supported(p);
+    // Accurate mode keeps the rounding of the SiLU*mul activations out of the result.  Where the w2 GEMM runs on the
+    // 64- / 128-row kernel, which waits on HBM, the activations are stored as fp16 (three more mantissa bits than
+    // bf16; clamped to the fp16 range) and the kernel turns its bf16 weight fragments into fp16 on their way to the
+    // MFMA: no extra traffic and no second pass.  Elsewhere they are a bf16 pair (value, residual) and both are
+    // multiplied (same pass in the streaming kernel, a second accumulating pass in the others).
+    const bool w2_on_mid = use_stream && T > kStreamW2MaxT && p.ksplit >= 2 && tile_mid_supported(p);
+    if (accurate && (w2_on_mid || (use_tile && T <= kTile128MaxT))) {
+        p.act_f16 = 1;
+        p.act_lo = nullptr;
+    }
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
         if (T <= kTile128MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
@@ -281,13 +292,13 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
-        if (use_stream && !accurate && T > kStreamW2MaxT && p.ksplit >= 2 && tile_mid_supported(p)) {
+        if (w2_on_mid) {
             rc = launch_gemm_tile_mid(p, seg_begin, 2, 64, s);
         } else if (use_stream) {
             rc = launch_gemm_stream(p, seg_begin, 2, s);  // multiplies act and act_lo in one pass
         } else {
             rc = use_tile ? tile_gemm(p, 2) : launch_gemm_generic(p, 2, s);
-            if (rc == 0 && accurate) {  // second pass: y += act_lo . w2
+            if (rc == 0 && accurate && !p.act_f16) {  // second pass: y += act_lo . w2
                 MoeProblem lo = p;
                 lo.act = p.act_lo;
                 lo.act_lo = nullptr;

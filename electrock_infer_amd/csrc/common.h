@@ -11,6 +11,7 @@ constexpr int kMaxExperts = 64;    // one lane per expert in the router / sort
 constexpr int kMaxTopK = 8;
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -44,9 +45,28 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
     __builtin_memcpy(&h, &v, 2);
     return h;
 }
+// fp16 with out-of-range values clamped to the largest finite one (a NaN stays a NaN)
+__device__ __forceinline__ uint16_t f32_to_f16_bits_sat(float f) {
+    const float c = fminf(fmaxf(f, -65504.0f), 65504.0f);
+    return f32_to_f16_bits(f != f ? f : c);
+}
 // two packed bf16 in one dword
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+// Eight bf16 as fp16: exact for every bf16 value of magnitude 2^-14 .. 65504 (fp16 has the longer mantissa); smaller
+// ones keep an absolute error below 2^-25, larger ones become the largest finite fp16.
+__device__ __forceinline__ f16x8_t bf16x8_to_f16x8(bf16x8_t v) {
+    u32x4_t w;
+    __builtin_memcpy(&w, &v, 16);
+    f16x8_t out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const auto h = __builtin_amdgcn_cvt_pkrtz(bf16_lo(w[i]), bf16_hi(w[i]));
+        out[2 * i] = h[0];
+        out[2 * i + 1] = h[1];
+    }
+    return out;
+}
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     bf16x2_t v;
@@ -113,6 +133,7 @@ struct MoeProblem {
     const uint16_t* w2;       // [E, H, I] bf16
     uint16_t* act;            // [sorted_len, I] bf16, rows in sorted (padded) order
     uint16_t* act_lo;         // same shape: bf16(value - act) in accurate mode, else null
+    int act_f16;              // act holds fp16 values (the other form of the accurate mode; act_lo is null then)
     int y_accumulate;         // w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
     const int32_t* sorted_ids;
@@ -127,6 +148,10 @@ struct MoeProblem {
 };
 // SiLU*mul result -> act (and the rounding residual -> act_lo in accurate mode)
 __device__ __forceinline__ void store_act(const MoeProblem& p, int64_t idx, float v) {
+    if (p.act_f16) {
+        p.act[idx] = f32_to_f16_bits_sat(v);
+        return;
+    }
     const uint16_t hi = f32_to_bf16_bits(v);
     p.act[idx] = hi;
     if (p.act_lo != nullptr) p.act_lo[idx] = f32_to_bf16_bits(v - bf16_bits_to_f32(hi));

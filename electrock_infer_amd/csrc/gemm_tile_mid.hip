@@ -66,7 +66,9 @@ __device__ __forceinline__ void wait_stages(int stages) {
 
 // One tile: `block` is the workgroup's index among those of its tile width, `col0` the first weight row
 // (MODE 1: first gate row) of the range that this width covers, `ntiles_n` the tiles across that range.
-template <int MODE, int MI, int NT>
+// F16 (w2 GEMM only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are converted on their
+// way from LDS to the MFMA, which costs this HBM-bound kernel nothing.
+template <int MODE, int MI, int NT, bool F16>
 __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __restrict__ seg_begin, int block, int col0,
                                           int ntiles_n, int kslice, uint8_t* smem) {
     typedef Geo<MI, NT> G;
@@ -202,6 +204,20 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
                     acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[set][f], fb[set][g], acc[f][g], 0, 0, 0);
             }
     };
+    auto multiply_f16 = [&](int set) {
+        f16x8_t hb[kCF];
+#pragma unroll
+        for (int g = 0; g < kCF; ++g) hb[g] = bf16x8_to_f16x8(fb[set][g]);
+#pragma unroll
+        for (int f = 0; f < kRF; ++f)
+            if (f < nfr) {
+                f16x8_t ha;
+                __builtin_memcpy(&ha, &fa[set][f], 16);
+#pragma unroll
+                for (int g = 0; g < kCF; ++g)
+                    acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ha, hb[g], acc[f][g], 0, 0, 0);
+            }
+    };
 
     // Stage st lives in ring slot st % kStages.  Stages are queued in order, so "at most n stages' worth of
     // copies in flight" means every stage but the n newest has landed.
@@ -213,7 +229,7 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
     for (int kt = 0; kt + 1 < nk; ++kt) {
         if (work) {
             read_frags(smem + buf * kStageBytes, 1, 1);
-            multiply(0);
+            if (F16) multiply_f16(0); else multiply(0);
         }
         {
             const int newer = nk - 2 - kt;  // stages queued after kt + 1: up to kt + kStages - 1, or the last one
@@ -225,13 +241,12 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
         buf = (buf + 1 == kStages) ? 0 : buf + 1;
         if (work) {
             read_frags(smem + buf * kStageBytes, 0, 0);
-            multiply(1);
+            if (F16) multiply_f16(1); else multiply(1);
         }
     }
     if (work) {
         read_frags(smem + buf * kStageBytes, 1, 1);
-        multiply(0);
-        multiply(1);
+        if (F16) { multiply_f16(0); multiply_f16(1); } else { multiply(0); multiply(1); }
     }
 
     // ---- epilogue through LDS (see the 256-row kernel).  Element i of lane (r16, kq) of a 16x16 accumulator is
@@ -250,7 +265,7 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
                     for (int i = 0; i < 4; ++i) {
                         const int row = wm * (32 * MI) + f * 16 + 4 * kq + i;
                         const float val = silu_mul(acc[f][gg][i], acc[f][gg + kCF / 2][i]);
-                        uint16_t bits = f32_to_bf16_bits(val);
+                        uint16_t bits = p.act_f16 ? f32_to_f16_bits_sat(val) : f32_to_bf16_bits(val);
                         if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
                         *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * (NT / 8) + gg * 16 + r16) * 2) = bits;
                     }
@@ -309,17 +324,17 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
     }
 }
 
-template <int MODE, int MI>
+template <int MODE, int MI, bool F16>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_mid_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
                                                                    int wide_blocks, int ntn_wide, int col0n,
                                                                    int ntn_narrow, int kslice) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int b = blockIdx.x;
-    if (b < wide_blocks) tile_body<MODE, MI, 256>(p, seg_begin, b, 0, ntn_wide, kslice, smem);
-    else tile_body<MODE, MI, 128>(p, seg_begin, b - wide_blocks, col0n, ntn_narrow, kslice, smem);
+    if (b < wide_blocks) tile_body<MODE, MI, 256, F16>(p, seg_begin, b, 0, ntn_wide, kslice, smem);
+    else tile_body<MODE, MI, 128, F16>(p, seg_begin, b - wide_blocks, col0n, ntn_narrow, kslice, smem);
 }
 
-template <int MODE, int MI>
+template <int MODE, int MI, bool F16>
 int launch_mid(const MoeProblem& p, const int32_t* seg_begin, hipStream_t s) {
     constexpr int kTM = 64 * MI;
     constexpr int kLdsBytes = Geo<MI, 256>::kLdsBytes > Geo<MI, 128>::kLdsBytes ? Geo<MI, 256>::kLdsBytes : Geo<MI, 128>::kLdsBytes;
@@ -344,12 +359,12 @@ int launch_mid(const MoeProblem& p, const int32_t* seg_begin, hipStream_t s) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_mid_kernel<MODE, MI>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_mid_kernel<MODE, MI, F16>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
         if (e != hipSuccess) return static_cast<int>(e);
         attr_set[dev] = true;
     }
-    hipLaunchKernelGGL((gemm_tile_mid_kernel<MODE, MI>), dim3(grid, static_cast<unsigned>(slices)), dim3(kThreads),
+    hipLaunchKernelGGL((gemm_tile_mid_kernel<MODE, MI, F16>), dim3(grid, static_cast<unsigned>(slices)), dim3(kThreads),
                        kLdsBytes, s, p, seg_begin, wide_blocks, ntn_wide, col0n, ntn_narrow,
                        (MODE == 1) ? p.H : p.I / p.ksplit);
     return launch_status();
@@ -366,8 +381,9 @@ bool tile_mid_supported(const MoeProblem& p) {
 // rows_per_tile: 64 or 128
 int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile, hipStream_t s) {
     if (!tile_mid_supported(p)) return EM_ERR_UNSUPPORTED;
-    if (rows_per_tile == 64) return mode == 1 ? launch_mid<1, 1>(p, seg_begin, s) : launch_mid<2, 1>(p, seg_begin, s);
-    return mode == 1 ? launch_mid<1, 2>(p, seg_begin, s) : launch_mid<2, 2>(p, seg_begin, s);
+    if (mode == 1) return rows_per_tile == 64 ? launch_mid<1, 1, false>(p, seg_begin, s) : launch_mid<1, 2, false>(p, seg_begin, s);
+    if (p.act_f16) return rows_per_tile == 64 ? launch_mid<2, 1, true>(p, seg_begin, s) : launch_mid<2, 2, true>(p, seg_begin, s);
+    return rows_per_tile == 64 ? launch_mid<2, 1, false>(p, seg_begin, s) : launch_mid<2, 2, false>(p, seg_begin, s);
 }
 
 }  // namespace em

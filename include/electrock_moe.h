@@ -44,7 +44,7 @@ extern "C" {
 
 /* em_moe_forward flags */
 #define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16      */
-#define EM_FLAG_ACCURATE       (1u << 1)  /* SiLU*mul activations kept as a bf16 hi+lo pair  */
+#define EM_FLAG_ACCURATE       (1u << 1)  /* SiLU*mul activations kept beyond one bf16       */
 #define EM_FLAG_GATE_F32_LOGITS (1u << 2) /* em_moe_forward_gated: route on the fp32 logits,   */
                                           /* not on their bf16 rounding                        */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
@@ -221,11 +221,15 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  *   w2            [E, H, I]   bf16 (mixtral_moe.py:75-79)
  *   out           [T, H]      bf16 (float32 with EM_FLAG_OUT_F32); may alias x
  *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k), 256-byte aligned
- * EM_FLAG_ACCURATE keeps the SiLU*mul activations as a bf16 pair (value, rounding
- * residual) and multiplies both with w2, which removes the one rounding the bf16 MFMA
- * of the w2 GEMM otherwise needs; together with EM_FLAG_OUT_F32 the result is within
- * fp32 accumulation error of the fp32 definition.  Costs ~14 % at T = 64 (no extra
- * weight traffic, more operand loads) and one extra w2 pass for T > 64.
+ * EM_FLAG_ACCURATE takes the one rounding to bf16 that the MFMA of the w2 GEMM
+ * otherwise needs out of the result.  From 9 to 352 tokens (the batch sizes at which
+ * the w2 GEMM waits on HBM) the SiLU*mul activations are kept as fp16, clamped to
+ * +-65504, and the kernel converts its bf16 weight fragments to fp16 on the way to
+ * the MFMA: mean relative error 2e-4, cost below 1 % up to 64 tokens, 4-6 % above.
+ * At the other sizes they are kept as a bf16 pair (value, rounding residual) and both
+ * are multiplied with w2: error at the level of fp32 accumulation; up to 8 tokens in
+ * the same pass (+6 %), above 352 tokens in a second pass over w2.  Both forms meet
+ * max-abs 2e-2 / mean relative 1e-3 against the fp32 definition with EM_FLAG_OUT_F32.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.
