@@ -43,8 +43,8 @@ def parse_args():
     ap.add_argument("--shape", choices=["8x7b", "8x22b"], default="8x7b",
                     help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
     ap.add_argument("--accurate", action="store_true",
-                    help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 or as a bf16 value + residual "
-                         "pair through the w2 GEMM instead of one bf16)")
+                    help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 instead of bf16 through the "
+                         "w2 GEMM)")
     ap.add_argument("--operands", choices=["gaussian", "zeros"], default="gaussian",
                     help="values of x and the expert weights.  'zeros' is a diagnostic: the matrix pipes then draw "
                          "little power and the same kernels run at the full shader clock, which separates the "
@@ -266,7 +266,7 @@ def main():
         for t in ((1, 8, 32, 64, 256) if args.shape == "8x7b" else (1, 64)):
             if t != T:
                 table.append(measure(torch, t, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2)))
-        if not args.accurate:  # the headline batch in accurate mode (activations kept beyond bf16)
+        if not args.accurate:  # the headline batch in accurate mode (fp16 activations)
             from electrock_infer_amd import _lib
             LayerRunner.base_flags = _lib.FLAG_ACCURATE
             r = measure(torch, T, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2))

@@ -271,13 +271,13 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     }
     const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
     const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T > kStreamMaxT && tile_supported(p);
-    // Accurate mode keeps the rounding of the SiLU*mul activations out of the result.  Where the w2 GEMM runs on the
-    // 64- / 128-row kernel, which waits on HBM, the activations are stored as fp16 (three more mantissa bits than
-    // bf16; clamped to the fp16 range) and the kernel turns its bf16 weight fragments into fp16 on their way to the
-    // MFMA: no extra traffic and no second pass.  Elsewhere they are a bf16 pair (value, residual) and both are
-    // multiplied (same pass in the streaming kernel, a second accumulating pass in the others).
+    // Accurate mode keeps the rounding of the SiLU*mul activations out of the result.  With the tuned kernels the
+    // activations are stored as fp16 (three more mantissa bits than bf16; clamped to the fp16 range) and the w2
+    // kernel turns its bf16 weight fragments into fp16 on their way to the MFMA: no extra traffic and no second
+    // pass.  The shape-generic kernels store a bf16 pair (value, residual) and multiply the residual in a second
+    // accumulating pass.
     const bool w2_on_mid = use_stream && T > kStreamW2MaxT && p.ksplit >= 2 && tile_mid_supported(p);
-    if (accurate && (w2_on_mid || (use_tile && T <= kTile128MaxT))) {
+    if (accurate && (use_stream || use_tile)) {
         p.act_f16 = 1;
         p.act_lo = nullptr;
     }
@@ -295,7 +295,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (w2_on_mid) {
             rc = launch_gemm_tile_mid(p, seg_begin, 2, 64, s);
         } else if (use_stream) {
-            rc = launch_gemm_stream(p, seg_begin, 2, s);  // multiplies act and act_lo in one pass
+            rc = launch_gemm_stream(p, seg_begin, 2, s);
         } else {
             rc = use_tile ? tile_gemm(p, 2) : launch_gemm_generic(p, 2, s);
             if (rc == 0 && accurate && !p.act_f16) {  // second pass: y += act_lo . w2
@@ -303,7 +303,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
                 lo.act = p.act_lo;
                 lo.act_lo = nullptr;
                 lo.y_accumulate = 1;
-                rc = use_tile ? tile_gemm(lo, 2) : launch_gemm_generic(lo, 2, s);
+                rc = launch_gemm_generic(lo, 2, s);  // (the tuned kernels never get here: they take fp16 activations)
             }
         }
         if (rc != 0) return rc;

@@ -132,9 +132,9 @@ struct MoeProblem {
     const uint16_t* w13;      // [E, 2I, H] bf16
     const uint16_t* w2;       // [E, H, I] bf16
     uint16_t* act;            // [sorted_len, I] bf16, rows in sorted (padded) order
-    uint16_t* act_lo;         // same shape: bf16(value - act) in accurate mode, else null
-    int act_f16;              // act holds fp16 values (the other form of the accurate mode; act_lo is null then)
-    int y_accumulate;         // w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
+    uint16_t* act_lo;         // same shape: bf16(value - act) in the accurate mode of the generic kernels, else null
+    int act_f16;              // act holds fp16 values (accurate mode of the tuned kernels; act_lo is null then)
+    int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
     const int32_t* sorted_ids;
     const int32_t* expert_ids;

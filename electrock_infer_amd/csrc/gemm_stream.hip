@@ -40,9 +40,9 @@ __device__ __forceinline__ u32x4_t ld16_stream(const uint16_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
 }
 
-// LO: the token rows exist as a bf16 pair act + act_lo (accurate mode, MODE 2 only); both halves are
-// multiplied with the same weight fragments, which costs no extra weight traffic.
-template <int MODE, bool LO>
+// F16 (accurate mode, MODE 2 only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are turned
+// into fp16 between the LDS tile and the MFMA, which costs this HBM-bound kernel nothing.
+template <int MODE, bool F16>
 __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem p,
                                                                      const int32_t* __restrict__ seg_begin,
                                                                      int tiles_per_expert, int kslice) {
@@ -93,8 +93,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 
         // token rows of this lane (operand layout: row r16 of each fragment)
         const uint16_t* arow[kMaxF];
-        int64_t lo_delta = 0;  // element offset from an act row to the same row of act_lo
-        if (LO) lo_delta = p.act_lo - p.act;
 #pragma unroll
         for (int f = 0; f < kMaxF; ++f) {
             arow[f] = nullptr;
@@ -115,7 +113,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 #pragma unroll
             for (int g = 0; g < 4; ++g) acc[f][g] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-        constexpr int kAW = LO ? 4 : 2;  // per fragment: two 32-wide K halves (x2 with the low parts)
+        constexpr int kAW = 2;  // per fragment: two 32-wide K halves
         u32x4_t b0[8], b1[8], a0[kMaxF][kAW], a1[kMaxF][kAW];
         auto issue = [&](int s, u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][kAW]) {
             const int koff = s * kStep;
@@ -126,7 +124,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
                     a[f][ks] = (arow[f] != nullptr) ? ld16(arow[f] + koff + ks * 32) : u32x4_t{0, 0, 0, 0};
-                    if (LO) a[f][2 + ks] = (arow[f] != nullptr) ? ld16(arow[f] + lo_delta + koff + ks * 32) : u32x4_t{0, 0, 0, 0};
                 }
         };
         auto consume = [&](u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][kAW]) {
@@ -136,19 +133,24 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 bf16x8_t bf[4];
+                f16x8_t hf[4];
 #pragma unroll
-                for (int g = 0; g < 4; ++g)
+                for (int g = 0; g < 4; ++g) {
                     bf[g] = *reinterpret_cast<const bf16x8_t*>(my + (g * 16 + r16) * kPitch + ks * 64 + kq * 16);
+                    if (F16) hf[g] = bf16x8_to_f16x8(bf[g]);
+                }
 #pragma unroll
                 for (int f = 0; f < kMaxF; ++f) {
                     if (f < nf) {
-                        bf16x8_t af;
-                        __builtin_memcpy(&af, &a[f][ks], 16);
+                        if (F16) {
+                            f16x8_t af;
+                            __builtin_memcpy(&af, &a[f][ks], 16);
 #pragma unroll
-                        for (int g = 0; g < 4; ++g)
-                            acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[g], acc[f][g], 0, 0, 0);
-                        if (LO) {
-                            __builtin_memcpy(&af, &a[f][2 + ks], 16);
+                            for (int g = 0; g < 4; ++g)
+                                acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, hf[g], acc[f][g], 0, 0, 0);
+                        } else {
+                            bf16x8_t af;
+                            __builtin_memcpy(&af, &a[f][ks], 16);
 #pragma unroll
                             for (int g = 0; g < 4; ++g)
                                 acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[g], acc[f][g], 0, 0, 0);
@@ -230,7 +232,7 @@ int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, 
     } else {
         const int tiles = p.H / kRows;
         const dim3 grid(static_cast<unsigned>(p.E * tiles), static_cast<unsigned>(p.ksplit));
-        if (p.act_lo != nullptr)
+        if (p.act_f16)
             hipLaunchKernelGGL((gemm_stream_kernel<2, true>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
         else
             hipLaunchKernelGGL((gemm_stream_kernel<2, false>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);

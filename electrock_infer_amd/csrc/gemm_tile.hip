@@ -64,7 +64,9 @@ constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, se
 
 // STREAM: the weight rows are copied with the non-temporal hint.  Right when most experts fit one row tile
 // (every weight byte is then read by one workgroup only); wrong when several row tiles share them through L2.
-template <int MODE, bool STREAM>
+// F16 (w2 GEMM in accurate mode): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
+// into fp16 once, before its first MFMA, and the fp16 MFMA of the same shape and rate runs instead.
+template <int MODE, bool STREAM, bool F16>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
                                                                int ntiles_n, int kslice) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -242,6 +244,22 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     // Unit u = 0..3 of a K step: row half h = u & 1 (fragments 4h .. 4h+3), K half k32 = u >> 1.
     // Token fragments live in register set u & 1, weight fragments (shared by both row halves) in set k32.
     bf16x8_t fa[2][4], fb[2][4];
+    auto mma = [](const bf16x8_t& a, const bf16x8_t& b, f32x4_t c) {
+        if (F16) {
+            f16x8_t ha, hb;  // the registers already hold fp16 bits
+            __builtin_memcpy(&ha, &a, 16);
+            __builtin_memcpy(&hb, &b, 16);
+            return __builtin_amdgcn_mfma_f32_16x16x32_f16(ha, hb, c, 0, 0, 0);
+        }
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    };
+    auto convert_weights = [&](int k32) {  // bf16 -> fp16 in place, once per fragment
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f16x8_t h = bf16x8_to_f16x8(fb[k32][g]);
+            __builtin_memcpy(&fb[k32][g], &h, 16);
+        }
+    };
     // operand fragments of unit u of K step stage_k (weight rows in ring slot bslot)
     // (nmi_tag: the wave's number of 32-row blocks as a constant, 0 = use the runtime value)
     auto read_frags = [&](int stage_k, int bslot, int u, auto nmi_tag) {
@@ -264,13 +282,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         constexpr bool FULL = NMI == 4;
         constexpr int reads = decltype(reads_tag)::value;
         const int h = u & 1, k32 = u >> 1;
+        if (F16 && h == 0) convert_weights(k32);  // unit u is the first to use the weight fragments of this K half
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (NMI ? (h * 4 + j < 2 * NMI) : (h * 4 + j < 2 * nmi)) {
 #pragma unroll
                 for (int gi = 0; gi < 4; ++gi) {
                     const int g = (j & 1) ? 3 - gi : gi;  // serpentine: one operand changes between neighbours
-                    acc[h * 4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[h][j], fb[k32][g], acc[h * 4 + j][g], 0, 0, 0);
+                    acc[h * 4 + j][g] = mma(fa[h][j], fb[k32][g], acc[h * 4 + j][g]);
                 }
             }
         if (FULL) {
@@ -327,7 +346,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             for (int i = 0; i < 16; ++i) {
                 const int j = i >> 2, g = (j & 1) ? 3 - (i & 3) : (i & 3);  // serpentine, as in multiply()
                 if (4 + j < 2 * NMI)
-                    acc[4 + j][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][j], fb[1][g], acc[4 + j][g], 0, 0, 0);
+                    acc[4 + j][g] = mma(fa[1][j], fb[1][g], acc[4 + j][g]);
                 const int n = i >> 1;
                 if ((i & 1) == 0) {
                     if (n < 4) { if (CA && (NMI == 4 || live[n])) copy_a(n, kt + 2); } else { if (CB) copy_b(n - 4, kt + 3, bs); }
@@ -399,7 +418,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     if (MODE == 1) {
         // act tile [256 rows][128 columns] bf16, row pitch 272 B
         constexpr int kPitchC = 128 * 2 + 16;
-        auto store_tile = [&](bool low_part) {
+        {
 #pragma unroll
             for (int f = 0; f < 8; ++f) {
                 if (f >= 2 * nmi) break;
@@ -411,13 +430,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                         const float g = acc[f][gg][i];
                         const float u = acc[f][gg + 2][i];
                         const float val = silu_mul(g, u);
-                        uint16_t bits = f32_to_bf16_bits(val);
-                        if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
+                        uint16_t bits = p.act_f16 ? f32_to_f16_bits_sat(val) : f32_to_bf16_bits(val);
                         *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = bits;
                     }
             }
             __syncthreads();
-            uint16_t* dst = low_part ? p.act_lo : p.act;
+            uint16_t* dst = p.act;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int c = tid + i * kThreads;  // 16-byte piece c of the tile: row c/16, columns (c%16)*8..+8
@@ -426,11 +444,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     *reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + nt * 128 + (c & 15) * 8) =
                         *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + (c & 15) * 16);
             }
-        };
-        store_tile(false);
-        if (p.act_lo != nullptr) {
-            __syncthreads();
-            store_tile(true);
         }
     } else {
         // slots of the tile's rows -> LDS; then per wave and 32-row fragment a private [32][64] fp32 tile, pitch 272 B
@@ -460,7 +473,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                 f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane & 15) * 16);
                 if (slot >= 0) {
                     f32x4_t* dst = reinterpret_cast<f32x4_t*>(ybase + static_cast<int64_t>(slot) * p.H + (lane & 15) * 4);
-                    if (p.y_accumulate) val += *dst;
                     *dst = val;
                 }
             }
@@ -497,10 +509,12 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev]) {
-        const void* kernels[4] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<1, true>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true>)};
+        const void* kernels[6] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, false>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<1, true, false>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, false>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, false>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, true>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, true>)};
         for (const void* k : kernels) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
             if (e != hipSuccess) return static_cast<int>(e);
@@ -510,18 +524,18 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     // one row tile per expert on average up to 7/8 full: weights are read once -> streaming copies
     const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * 7;
     const dim3 grid1(grid, 1), grid2(grid, static_cast<unsigned>(p.ksplit));
+    auto go = [&](auto kernel, dim3 g, int kslice) {
+        hipLaunchKernelGGL(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice);
+    };
     if (mode == 1) {
-        if (stream_b)
-            hipLaunchKernelGGL((gemm_tile_kernel<1, true>), grid1, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, p.H);
-        else
-            hipLaunchKernelGGL((gemm_tile_kernel<1, false>), grid1, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, p.H);
+        if (stream_b) go(gemm_tile_kernel<1, true, false>, grid1, p.H);
+        else go(gemm_tile_kernel<1, false, false>, grid1, p.H);
+    } else if (p.act_f16) {
+        if (stream_b) go(gemm_tile_kernel<2, true, true>, grid2, p.I / p.ksplit);
+        else go(gemm_tile_kernel<2, false, true>, grid2, p.I / p.ksplit);
     } else {
-        if (stream_b)
-            hipLaunchKernelGGL((gemm_tile_kernel<2, true>), grid2, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n,
-                               p.I / p.ksplit);
-        else
-            hipLaunchKernelGGL((gemm_tile_kernel<2, false>), grid2, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n,
-                               p.I / p.ksplit);
+        if (stream_b) go(gemm_tile_kernel<2, true, false>, grid2, p.I / p.ksplit);
+        else go(gemm_tile_kernel<2, false, false>, grid2, p.I / p.ksplit);
     }
     return launch_status();
 }

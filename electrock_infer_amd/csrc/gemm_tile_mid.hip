@@ -255,7 +255,7 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
     if (MODE == 1) {
         constexpr int kColsC = NT / 2;  // act columns of the tile
         constexpr int kPitchC = kColsC * 2 + 16;
-        auto store_tile = [&](bool low_part) {
+        {
 #pragma unroll
             for (int f = 0; f < kRF; ++f) {
                 if (f >= nfr) break;
@@ -266,12 +266,11 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
                         const int row = wm * (32 * MI) + f * 16 + 4 * kq + i;
                         const float val = silu_mul(acc[f][gg][i], acc[f][gg + kCF / 2][i]);
                         uint16_t bits = p.act_f16 ? f32_to_f16_bits_sat(val) : f32_to_bf16_bits(val);
-                        if (low_part) bits = f32_to_bf16_bits(val - bf16_bits_to_f32(bits));
                         *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * (NT / 8) + gg * 16 + r16) * 2) = bits;
                     }
             }
             __syncthreads();
-            uint16_t* dst = low_part ? p.act_lo : p.act;
+            uint16_t* dst = p.act;
             constexpr int kPiecesRow = kColsC / 8;  // 16-byte pieces per row
 #pragma unroll
             for (int i = 0; i < kTM * kPiecesRow / kThreads; ++i) {
@@ -281,11 +280,6 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
                     *reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + col0 + nt * kColsC + pc * 8) =
                         *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + pc * 16);
             }
-        };
-        store_tile(false);
-        if (p.act_lo != nullptr) {
-            __syncthreads();
-            store_tile(true);
         }
     } else {
         constexpr int kColsY = NT / 4;          // fp32 columns of a wave
@@ -315,7 +309,6 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
                 f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane % kLanesRow) * 16);
                 if (slot >= 0) {
                     f32x4_t* dst = reinterpret_cast<f32x4_t*>(ybase + static_cast<int64_t>(slot) * p.H + (lane % kLanesRow) * 4);
-                    if (p.y_accumulate) val += *dst;
                     *dst = val;
                 }
             }

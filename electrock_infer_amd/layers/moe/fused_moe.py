@@ -107,8 +107,7 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     ``hidden_states`` and that tensor is returned, as in the reference.
     ``out_dtype=torch.float32`` returns the un-rounded fp32 result instead
     (not available together with ``inplace``).  ``accurate=True`` keeps the
-    SiLU*mul activations beyond one bf16 through the w2 GEMM (fp16 where that is
-    free, a bf16 value + residual pair elsewhere).
+    SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM.
     """
     if activation != "silu":
         raise NotImplementedError(f"Activation {activation} not supported.")

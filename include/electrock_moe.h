@@ -222,14 +222,14 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  *   out           [T, H]      bf16 (float32 with EM_FLAG_OUT_F32); may alias x
  *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k), 256-byte aligned
  * EM_FLAG_ACCURATE takes the one rounding to bf16 that the MFMA of the w2 GEMM
- * otherwise needs out of the result.  From 9 to 352 tokens (the batch sizes at which
- * the w2 GEMM waits on HBM) the SiLU*mul activations are kept as fp16, clamped to
- * +-65504, and the kernel converts its bf16 weight fragments to fp16 on the way to
- * the MFMA: mean relative error 2e-4, cost below 1 % up to 64 tokens, 4-6 % above.
- * At the other sizes they are kept as a bf16 pair (value, rounding residual) and both
- * are multiplied with w2: error at the level of fp32 accumulation; up to 8 tokens in
- * the same pass (+6 %), above 352 tokens in a second pass over w2.  Both forms meet
- * max-abs 2e-2 / mean relative 1e-3 against the fp32 definition with EM_FLAG_OUT_F32.
+ * otherwise needs out of the result: the SiLU*mul activations are kept as fp16,
+ * clamped to +-65504, and the w2 kernel converts its bf16 weight fragments to fp16
+ * on the way to the MFMA.  Mean relative error 2e-4 instead of 1.7e-3; no cost in
+ * time up to 64 tokens, 4-6 % above (at 8192 tokens: +10 % on the w2 GEMM).  For
+ * shapes only the generic kernels take, the activations are kept as a bf16 pair
+ * (value, rounding residual) and the residual is multiplied in a second pass over
+ * w2.  Both forms meet max-abs 2e-2 / mean relative 1e-3 against the fp32 definition
+ * with EM_FLAG_OUT_F32.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.
