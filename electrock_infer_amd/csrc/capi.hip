@@ -224,6 +224,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     const bool accurate = (flags & EM_FLAG_ACCURATE) != 0;
     p.act_lo = accurate ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
     p.act_f16 = 0;
+    p.y_f16 = 0;
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
@@ -281,6 +282,10 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         p.act_f16 = 1;
         p.act_lo = nullptr;
     }
+    // Where the output is bf16, the partial results of the 256-row w2 kernel are fp16 (their rounding, 2^-12, is far
+    // below the output's, 2^-9): half the bytes written by the kernel's epilogues, which all fall into the same
+    // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer).
+    if (use_tile && T > kTile128MaxT && !(flags & EM_FLAG_OUT_F32)) p.y_f16 = 1;
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
         if (T <= kTile128MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);

@@ -67,6 +67,10 @@ __device__ __forceinline__ f16x8_t bf16x8_to_f16x8(bf16x8_t v) {
     }
     return out;
 }
+// two floats as packed fp16 (round to nearest even; clamped to the fp16 range)
+__device__ __forceinline__ uint32_t pack_f16_sat(float lo, float hi) {
+    return static_cast<uint32_t>(f32_to_f16_bits_sat(lo)) | (static_cast<uint32_t>(f32_to_f16_bits_sat(hi)) << 16);
+}
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     bf16x2_t v;
@@ -136,6 +140,7 @@ struct MoeProblem {
     int act_f16;              // act holds fp16 values (accurate mode of the tuned kernels; act_lo is null then)
     int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
+    int y_f16;                // y holds fp16 values instead (256-row kernel with a bf16 layer output)
     const int32_t* sorted_ids;
     const int32_t* expert_ids;
     const int32_t* post_pad;

@@ -188,7 +188,8 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(MoeProblem p) {
 // out[t, :] = sum_j w[t, j] * sum_z y[z, t*k + j, :]   (fp32, one final rounding)
 // kStream: the partial results are too many to still sit in the caches when they are read (exactly once):
 // streaming loads.  Small sets are read back out of L2, where streaming loads of just-written lines are slower.
-template <bool kOutF32, bool kStream>
+// kYF16: the partial results are fp16.
+template <bool kOutF32, bool kStream, bool kYF16>
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
                                                       void* __restrict__ out, int64_t T, int H, int top_k,
                                                       int ksplit) {
@@ -198,13 +199,19 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < top_k; ++j) {
             const float wj = w[t * top_k + j];
-            const float* row = y + (t * top_k + j) * static_cast<int64_t>(H) + h;
-            auto load = [](const float* ptr) {
-                return kStream ? __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(ptr))
-                               : *reinterpret_cast<const f32x4_t*>(ptr);
+            const int64_t at = (t * top_k + j) * static_cast<int64_t>(H) + h;
+            auto load = [&](int64_t idx) {
+                if (kYF16) {
+                    const u32x2_t* ptr = reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(y) + idx);
+                    const u32x2_t v = kStream ? __builtin_nontemporal_load(ptr) : *ptr;
+                    return f32x4_t{f16_bits_to_f32(static_cast<uint16_t>(v[0])), f16_bits_to_f32(static_cast<uint16_t>(v[0] >> 16)),
+                                   f16_bits_to_f32(static_cast<uint16_t>(v[1])), f16_bits_to_f32(static_cast<uint16_t>(v[1] >> 16))};
+                }
+                const f32x4_t* ptr = reinterpret_cast<const f32x4_t*>(y + idx);
+                return kStream ? __builtin_nontemporal_load(ptr) : *ptr;
             };
-            f32x4_t s = load(row);
-            for (int z = 1; z < ksplit; ++z) s += load(row + z * zstride);
+            f32x4_t s = load(at);
+            for (int z = 1; z < ksplit; ++z) s += load(at + z * zstride);
             acc += wj * s;
         }
         if (kOutF32) {
@@ -245,12 +252,13 @@ int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
     const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 1024));
     const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
     // beyond the memory-side cache (256 MB) the partial results come back from HBM
-    const bool stream = static_cast<int64_t>(p.ksplit) * p.T * p.top_k * p.H * 4 > (int64_t{256} << 20);
+    const bool stream = static_cast<int64_t>(p.ksplit) * p.T * p.top_k * p.H * (p.y_f16 ? 2 : 4) > (int64_t{256} << 20);
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k, p.ksplit);
     };
-    if (out_f32) { if (stream) go(combine_kernel<true, true>); else go(combine_kernel<true, false>); }
-    else { if (stream) go(combine_kernel<false, true>); else go(combine_kernel<false, false>); }
+    if (out_f32) { if (stream) go(combine_kernel<true, true, false>); else go(combine_kernel<true, false, false>); }
+    else if (p.y_f16) { if (stream) go(combine_kernel<false, true, true>); else go(combine_kernel<false, false, true>); }
+    else { if (stream) go(combine_kernel<false, true, false>); else go(combine_kernel<false, false, false>); }
     return launch_status();
 }
 

@@ -452,7 +452,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         uint8_t* ytile = smem + 1024 + wave * (32 * kPitchY);
         if (tid < kTM) slots[tid] = my_slot;
         __syncthreads();
-        float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
+        const int64_t yoff = static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
+        float* ybase = p.y + yoff;
+        uint16_t* ybase_h = reinterpret_cast<uint16_t*>(p.y) + yoff;  // the same partial results as fp16 (p.y_f16)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
             if (mi >= nmi) break;
@@ -472,8 +474,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                 const int slot = slots[wm * 128 + mi * 32 + row];
                 f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane & 15) * 16);
                 if (slot >= 0) {
-                    f32x4_t* dst = reinterpret_cast<f32x4_t*>(ybase + static_cast<int64_t>(slot) * p.H + (lane & 15) * 4);
-                    *dst = val;
+                    const int64_t at = static_cast<int64_t>(slot) * p.H + (lane & 15) * 4;
+                    if (p.y_f16)
+                        *reinterpret_cast<u32x2_t*>(ybase_h + at) = u32x2_t{pack_f16_sat(val[0], val[1]), pack_f16_sat(val[2], val[3])};
+                    else
+                        *reinterpret_cast<f32x4_t*>(ybase + at) = val;
                 }
             }
             __builtin_amdgcn_wave_barrier();

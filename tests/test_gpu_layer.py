@@ -9,12 +9,13 @@ fp32 result to bf16 alone costs about 1.4e-3 mean relative error and up to
 half a bf16 ulp (0.0156 for |v| in [4, 8), 0.031 for [8, 16)) — so every case
 reports the measured errors of the fp32 output and of the bf16 output, and
 asserts
-    accurate    : (EM_FLAG_ACCURATE, fp32 output: activations kept as a bf16 hi+lo pair)
+    accurate    : (EM_FLAG_ACCURATE, fp32 output: activations kept as fp16 instead of bf16)
                   the stated target itself, max_abs <= 2e-2 and mean_rel <= 1e-3
     fp32 output : mean_rel <= TOL_MEAN_REL_F32, max_abs <= TOL_MAX_ABS_F32 * max|ref|
                   (the activation rounding is a relative error, so the bound scales
                   with the output magnitude: max|ref| is ~9 at 8x7B and ~16 at 8x22B)
-    bf16 output : equal to the rounded fp32 output within 1 bf16 ulp, and
+    bf16 output : equal to the rounded fp32 output within 1 bf16 ulp (above 352 tokens: plus
+                  2^-10 of max|ref| for the rounding of the fp16 partial results), and
                   mean_rel <= TOL_MEAN_REL_BF16
 """
 import json
@@ -62,7 +63,8 @@ def check_routing(ws, lg_cpu_f32, T, E=8, k=2):
     assert np.array_equal(e[:me], oe[:me]) and (e[me:] == 0).all()
 
 
-def check_outputs(case, out_f32, out_bf16, ref, out_acc=None):
+def check_outputs(case, out_f32, out_bf16, ref, out_acc=None, tokens=None):
+    """tokens: batch size of the call when only some of its rows are checked."""
     f = error_stats(out_f32, ref)
     b = error_stats(out_bf16.float(), ref)
     a = error_stats(out_acc, ref) if out_acc is not None else None
@@ -71,9 +73,16 @@ def check_outputs(case, out_f32, out_bf16, ref, out_acc=None):
         assert a["max_abs"] <= TARGET_MAX_ABS and a["mean_rel"] <= TARGET_MEAN_REL, (case, a)
     assert f["mean_rel"] <= TOL_MEAN_REL_F32 and f["max_abs"] <= TOL_MAX_ABS_F32 * float(ref.abs().max()), (case, f)
     assert b["mean_rel"] <= TOL_MEAN_REL_BF16, (case, b)
+    # The bf16 output is the fp32 output rounded once.  Above 352 tokens the bf16-output path keeps the partial
+    # results of the w2 GEMM as fp16 (relative step 2^-11, against 2^-8 of the output format): where the partial
+    # results cancel, their rounding shows in absolute terms: at most 2^-11 of each partial result (measured: up to
+    # 0.33 * 2^-10 * max|ref|); asserted with max|ref| standing for the largest partial result.
     rounded = out_f32.to(torch.bfloat16).float()
     ulp = torch.maximum(rounded.abs(), torch.tensor(1e-30, device=rounded.device)) * 2.0 ** -7
-    assert ((out_bf16.float() - rounded).abs() <= ulp).all()
+    excess = ((out_bf16.float() - rounded).abs() - ulp).clamp_min(0)
+    slack = 0.0 if (tokens or out_f32.shape[0]) <= 352 else 2.0 ** -10 * float(ref.abs().max())
+    record(case + "_bf16_vs_rounded_f32", max_excess_over_1ulp=float(excess.max()), allowed=slack)
+    assert float(excess.max()) <= slack
 
 
 def run_both(x, lg, w13, w2, flags=0):
@@ -147,7 +156,7 @@ def test_layer_8x7b_decode(mixtral_8x7b, T):
     check_routing(get_workspace(DEV, T, 4096, 14336, 8, 2), lg.float().cpu(), T)
     rows = list(range(T)) if T <= 64 else list(range(0, T, 4))
     ref = oracle_rows(x, lg, m["w13_cpu"], m["w2_cpu"], rows)
-    check_outputs(f"8x7b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_acc[rows].cpu())
+    check_outputs(f"8x7b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_acc[rows].cpu(), tokens=T)
 
 
 @pytest.mark.parametrize("logits", ["normal", "zipf", "two_experts"])
@@ -170,7 +179,7 @@ def test_layer_8x7b_prefill(mixtral_8x7b, logits):
     check_routing(get_workspace(DEV, T, 4096, 14336, 8, 2), lg.float().cpu(), T)
     rows = torch.randperm(T, generator=g)[:96].tolist() + [0, T - 1]
     ref = oracle_rows(m["x"], lg, m["w13_cpu"], m["w2_cpu"], rows)
-    check_outputs(f"8x7b_prefill_{logits}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_acc[rows].cpu())
+    check_outputs(f"8x7b_prefill_{logits}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_acc[rows].cpu(), tokens=8192)
     # size-independent properties on the full result
     assert torch.isfinite(out_f32).all()
     perm = torch.randperm(T, generator=g).to(DEV)     # token-wise layer: permuting tokens permutes outputs
@@ -192,7 +201,7 @@ def test_layer_8x22b_shape():
         check_routing(get_workspace(DEV, T, 6144, 16384, 8, 2), lt.float().cpu(), T)
         rows = list(range(T)) if T <= 64 else list(range(0, T, 64))
         ref = oracle_rows(xt, lt, w13_cpu, w2_cpu, rows)
-        check_outputs(f"8x22b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_acc[rows].cpu())
+        check_outputs(f"8x22b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_acc[rows].cpu(), tokens=T)
 
 
 def test_fusedmoe_module_runs_in_place_and_matches(mixtral_8x7b):
