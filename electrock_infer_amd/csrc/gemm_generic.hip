@@ -188,8 +188,7 @@ __global__ __launch_bounds__(kThreads) void gemm_generic_kernel(MoeProblem p) {
 // out[t, :] = sum_j w[t, j] * sum_z y[z, t*k + j, :]   (fp32, one final rounding)
 // kStream: the partial results are too many to still sit in the caches when they are read (exactly once):
 // streaming loads.  Small sets are read back out of L2, where streaming loads of just-written lines are slower.
-// kYF16: the partial results are fp16.
-template <bool kOutF32, bool kStream, bool kYF16>
+template <bool kOutF32, bool kStream>
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
                                                       void* __restrict__ out, int64_t T, int H, int top_k,
                                                       int ksplit) {
@@ -199,19 +198,13 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < top_k; ++j) {
             const float wj = w[t * top_k + j];
-            const int64_t at = (t * top_k + j) * static_cast<int64_t>(H) + h;
-            auto load = [&](int64_t idx) {
-                if (kYF16) {
-                    const u32x2_t* ptr = reinterpret_cast<const u32x2_t*>(reinterpret_cast<const uint16_t*>(y) + idx);
-                    const u32x2_t v = kStream ? __builtin_nontemporal_load(ptr) : *ptr;
-                    return f32x4_t{f16_bits_to_f32(static_cast<uint16_t>(v[0])), f16_bits_to_f32(static_cast<uint16_t>(v[0] >> 16)),
-                                   f16_bits_to_f32(static_cast<uint16_t>(v[1])), f16_bits_to_f32(static_cast<uint16_t>(v[1] >> 16))};
-                }
-                const f32x4_t* ptr = reinterpret_cast<const f32x4_t*>(y + idx);
-                return kStream ? __builtin_nontemporal_load(ptr) : *ptr;
+            const float* row = y + (t * top_k + j) * static_cast<int64_t>(H) + h;
+            auto load = [](const float* ptr) {
+                return kStream ? __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(ptr))
+                               : *reinterpret_cast<const f32x4_t*>(ptr);
             };
-            f32x4_t s = load(at);
-            for (int z = 1; z < ksplit; ++z) s += load(at + z * zstride);
+            f32x4_t s = load(row);
+            for (int z = 1; z < ksplit; ++z) s += load(row + z * zstride);
             acc += wj * s;
         }
         if (kOutF32) {
@@ -220,6 +213,37 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
             u32x2_t o = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3])};
             *reinterpret_cast<u32x2_t*>(static_cast<uint16_t*>(out) + t * H + h) = o;
         }
+    }
+}
+
+// The same sum over fp16 partial results, bf16 out: eight columns per thread (16-byte loads and stores).
+template <bool kStream>
+__global__ __launch_bounds__(256) void combine_f16_kernel(const uint16_t* __restrict__ y, const float* __restrict__ w,
+                                                          uint16_t* __restrict__ out, int64_t T, int H, int top_k,
+                                                          int ksplit) {
+    const int64_t t = blockIdx.x;
+    const int64_t zstride = T * top_k * static_cast<int64_t>(H);
+    for (int h = (blockIdx.y * 256 + threadIdx.x) * 8; h < H; h += gridDim.y * 256 * 8) {
+        float acc[8] = {};
+        for (int j = 0; j < top_k; ++j) {
+            const float wj = w[t * top_k + j];
+            const uint16_t* row = y + (t * top_k + j) * static_cast<int64_t>(H) + h;
+            float s[8] = {};
+            for (int z = 0; z < ksplit; ++z) {
+                const u32x4_t* ptr = reinterpret_cast<const u32x4_t*>(row + z * zstride);
+                const u32x4_t v = kStream ? __builtin_nontemporal_load(ptr) : *ptr;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s[2 * i] += f16_bits_to_f32(static_cast<uint16_t>(v[i]));
+                    s[2 * i + 1] += f16_bits_to_f32(static_cast<uint16_t>(v[i] >> 16));
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] += wj * s[i];
+        }
+        const u32x4_t o = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]),
+                           pack_bf16(acc[6], acc[7])};
+        *reinterpret_cast<u32x4_t*>(out + t * H + h) = o;
     }
 }
 
@@ -249,16 +273,26 @@ int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s) {
 
 int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
     if (p.T == 0) return 0;
-    const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 1024));
-    const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
     // beyond the memory-side cache (256 MB) the partial results come back from HBM
     const bool stream = static_cast<int64_t>(p.ksplit) * p.T * p.top_k * p.H * (p.y_f16 ? 2 : 4) > (int64_t{256} << 20);
+    if (p.y_f16) {  // bf16 out only
+        if (out_f32 || p.H % 8 != 0) return EM_ERR_UNSUPPORTED;
+        const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 2048));
+        const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
+        auto go = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.topk_w,
+                               static_cast<uint16_t*>(out), p.T, p.H, p.top_k, p.ksplit);
+        };
+        if (stream) go(combine_f16_kernel<true>); else go(combine_f16_kernel<false>);
+        return launch_status();
+    }
+    const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 1024));
+    const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k, p.ksplit);
     };
-    if (out_f32) { if (stream) go(combine_kernel<true, true, false>); else go(combine_kernel<true, false, false>); }
-    else if (p.y_f16) { if (stream) go(combine_kernel<false, true, true>); else go(combine_kernel<false, false, true>); }
-    else { if (stream) go(combine_kernel<false, true, false>); else go(combine_kernel<false, false, false>); }
+    if (out_f32) { if (stream) go(combine_kernel<true, true>); else go(combine_kernel<true, false>); }
+    else { if (stream) go(combine_kernel<false, true>); else go(combine_kernel<false, false>); }
     return launch_status();
 }
 
