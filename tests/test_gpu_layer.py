@@ -293,6 +293,22 @@ def test_layer_router_and_sort_in_one_launch(T, dtype):
     check_routing(get_workspace(DEV, T, 256, 512, 8, 2), lg.float(), T)
 
 
+@pytest.mark.parametrize("T", [7, 64, 300, 777])
+def test_layer_accurate_mode_with_bf16_output(T):
+    """Accurate mode is asserted against the stated target with an fp32 output everywhere else; with the default bf16
+    output (fp16 activations, and above 352 tokens fp16 partial results as well) the result is that fp32 output
+    rounded once, up to the rounding of the partial results."""
+    announce(f"layer accurate mode, bf16 out T={T}")
+    x, lg, w13, w2 = (t.to(DEV) for t in O.make_inputs(T, MID["H"], MID["I"], seed=7 * T))
+    acc_f32 = run_accurate(x, lg, w13, w2)
+    acc_bf16 = fused_experts(x, w13, w2, lg, 2, renormalize=True, accurate=True)
+    assert acc_bf16.dtype == torch.bfloat16
+    rounded = acc_f32.to(torch.bfloat16).float()
+    ulp = rounded.abs().clamp_min(1e-30) * 2.0 ** -7
+    slack = 0.0 if T <= 352 else 2.0 ** -10 * float(acc_f32.abs().max())
+    assert float(((acc_bf16.float() - rounded).abs() - ulp).max()) <= slack
+
+
 @pytest.mark.parametrize("T", [96, 300])
 def test_layer_mid_kernel_wide_w13_tiles(T):
     """I = 4096 makes 8 experts x 32 column tiles = one full round of CUs, so the w13 GEMM of the 64- and
