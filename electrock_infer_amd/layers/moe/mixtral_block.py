@@ -39,25 +39,27 @@ class ReplicatedLinear(nn.Module):
 class MixtralMoE(nn.Module):
     """``forward(hidden_states)`` = ``experts(hidden_states, gate(hidden_states))`` of the reference
     (models/mixtral.py:53-63), with the gate computed inside the router's launch.  ``bf16_logits=True``
-    (default) rounds the logits to bf16 before the selection as the reference's bf16 gate does."""
+    (default) rounds the logits to bf16 before the selection as the reference's bf16 gate does; ``accurate=True``
+    keeps the SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM."""
 
     def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int,
                  params_dtype: Optional[torch.dtype] = None, tp_size: Optional[int] = None, prefix: str = "",
-                 bf16_logits: bool = True):
+                 bf16_logits: bool = True, accurate: bool = False):
         super().__init__()
         self.hidden_size = hidden_size
         self.bf16_logits = bf16_logits
         self.gate = ReplicatedLinear(hidden_size, num_experts, bias=False, params_dtype=params_dtype)
         self.experts = FusedMoE(num_experts=num_experts, top_k=top_k, hidden_size=hidden_size,
                                 intermediate_size=intermediate_size, params_dtype=params_dtype,
-                                reduce_results=True, renormalize=True, tp_size=tp_size)
+                                reduce_results=True, renormalize=True, tp_size=tp_size, accurate=accurate)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         orig_shape = hidden_states.shape
         hidden_states = hidden_states.view(-1, self.hidden_size)
         e = self.experts
         out = fused_experts_gated(hidden_states, self.gate.weight, e.w13_weight, e.w2_weight, topk=e.top_k,
-                                  renormalize=e.renormalize, inplace=True, bf16_logits=self.bf16_logits)
+                                  renormalize=e.renormalize, inplace=True, bf16_logits=self.bf16_logits,
+                                  accurate=e.accurate)
         if e.reduce_results and e.tp_size > 1:
             dist.all_reduce(out)
         return out.view(orig_shape)
@@ -83,7 +85,7 @@ class PostAttentionMoE(nn.Module):
         orig_shape = hidden_states.shape
         out, res = fused_experts_normed(hidden_states.view(-1, moe.hidden_size), residual.view(-1, moe.hidden_size),
                                         norm.weight, norm.eps, moe.gate.weight, e.w13_weight, e.w2_weight, topk=e.top_k,
-                                        renormalize=e.renormalize, bf16_logits=moe.bf16_logits)
+                                        renormalize=e.renormalize, bf16_logits=moe.bf16_logits, accurate=e.accurate)
         if e.reduce_results and e.tp_size > 1:
             dist.all_reduce(out)
         return out.view(orig_shape), res.view(orig_shape)

@@ -217,6 +217,10 @@ def test_fusedmoe_module_runs_in_place_and_matches(mixtral_8x7b):
     ret = layer(x, lg)
     assert ret.data_ptr() == x.data_ptr()            # the input tensor is overwritten and returned
     assert torch.equal(ret, expect)
+    layer.accurate = True                            # the keyword-only option of this build
+    x2 = m["x"][:48].clone()
+    expect = fused_experts(x2.clone(), m["w13"], m["w2"], lg, 2, renormalize=True, accurate=True)
+    assert torch.equal(layer(x2, lg), expect) and not torch.equal(expect, ret)
 
 
 def test_dense_equals_sparse_when_one_expert_wins():

@@ -22,9 +22,13 @@ def test_op_surface_matches_reference_binding():
     assert list(inspect.signature(fused_experts).parameters)[:8] == [
         "hidden_states", "w1", "w2", "gating_output", "topk", "renormalize", "inplace", "activation"]
     assert list(inspect.signature(fused_topk).parameters) == ["hidden_states", "gating_output", "topk", "renormalize"]
-    assert list(inspect.signature(FusedMoE.__init__).parameters)[1:] == [
+    params = inspect.signature(FusedMoE.__init__).parameters
+    assert list(params)[1:9] == [
         "num_experts", "top_k", "hidden_size", "intermediate_size", "tp_size", "params_dtype", "renormalize",
         "reduce_results"]
+    # the one addition is keyword-only and off by default
+    assert list(params)[9:] == ["accurate"] and params["accurate"].kind is inspect.Parameter.KEYWORD_ONLY
+    assert params["accurate"].default is False
     assert em._C is _C
 
 
