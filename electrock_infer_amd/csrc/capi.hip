@@ -25,6 +25,7 @@ constexpr int64_t kStreamW2MaxT = 8;
 // 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 352 tokens.
 constexpr int64_t kTile64MaxT = 192;
 constexpr int64_t kTile128MaxT = 352;
+constexpr int64_t kTile128W2MaxT = 448;  // the w2 GEMM stays on 128-row tiles a little longer (156-160 against 165 us)
 
 // Rows per sorted block, the counterpart of _get_moe_config (fused_moe.py:327-339):
 // 16 (one MFMA fragment) for the streaming kernel, 32 for the tiled kernel, which cuts
@@ -285,10 +286,10 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     // Where the output is bf16, the partial results of the 256-row w2 kernel are fp16 (their rounding, 2^-12, is far
     // below the output's, 2^-9): half the bytes written by the kernel's epilogues, which all fall into the same
     // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer).
-    if (use_tile && T > kTile128MaxT && !(flags & EM_FLAG_OUT_F32)) p.y_f16 = 1;
+    if (use_tile && T > kTile128W2MaxT && !(flags & EM_FLAG_OUT_F32)) p.y_f16 = 1;
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
-        if (T <= kTile128MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
+        if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
         return launch_gemm_tile(q, seg_begin, mode, s);
     };
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
