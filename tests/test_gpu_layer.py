@@ -313,6 +313,25 @@ def test_layer_accurate_mode_with_bf16_output(T):
     assert float(((acc_bf16.float() - rounded).abs() - ulp).max()) <= slack
 
 
+@pytest.mark.parametrize("E,k", [(4, 1), (16, 4), (64, 8)])
+@pytest.mark.parametrize("T", [9, 70, 500])
+def test_layer_other_expert_counts(T, E, k):
+    """The path is built for 8 experts and top-2; other counts go through the same kernels (streaming, 64- / 128-row
+    and 256-row tiles) with the two-launch routing front."""
+    announce(f"layer E={E} top-{k} T={T}")
+    x, lg, w13, w2 = O.make_inputs(T, 256, 512, E=E, seed=T + E)
+    ref = O.moe_layer_fp32(x, lg, w13, w2, topk=k)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out = fused_experts(xd, w13d, w2d, lgd, k, renormalize=True, out_dtype=torch.float32)
+    check_routing(get_workspace(DEV, T, 256, 512, E, k), lg.float(), T, E=E, k=k)
+    st = error_stats(out.cpu(), ref)
+    record(f"E{E}_k{k}_T{T}", f32=st)
+    assert st["mean_rel"] <= TOL_MEAN_REL_F32 and st["max_abs"] <= TOL_MAX_ABS_F32 * float(ref.abs().max()), st
+    acc = fused_experts(xd, w13d, w2d, lgd, k, renormalize=True, out_dtype=torch.float32, accurate=True)
+    sa = error_stats(acc.cpu(), ref)
+    assert sa["max_abs"] <= TARGET_MAX_ABS and sa["mean_rel"] <= TARGET_MEAN_REL, sa
+
+
 @pytest.mark.parametrize("T", [96, 300])
 def test_layer_mid_kernel_wide_w13_tiles(T):
     """I = 4096 makes 8 experts x 32 column tiles = one full round of CUs, so the w13 GEMM of the 64- and
