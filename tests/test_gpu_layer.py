@@ -313,6 +313,25 @@ def test_layer_accurate_mode_with_bf16_output(T):
     assert float(((acc_bf16.float() - rounded).abs() - ulp).max()) <= slack
 
 
+@pytest.mark.parametrize("routing", ["normal", "one_expert"])
+@pytest.mark.parametrize("T", [40, 100, 300, 600, 1500])
+def test_layer_column_tiles_not_a_multiple_of_eight(T, routing):
+    """H = 768 and I = 1152 give 3 and 9 column tiles: the tile orders that do not deal whole columns to the XCDs,
+    and launches of the 64- / 128-row kernel whose tile count fills no whole round."""
+    announce(f"layer H=768 I=1152 T={T} {routing}")
+    x, lg, w13, w2 = O.make_inputs(T, 768, 1152, seed=3 * T)
+    if routing == "one_expert":
+        lg = lg.float()
+        lg[:, 5] += 30.0
+        lg = lg.to(torch.bfloat16)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out_f32, out_bf16 = run_both(xd, lgd, w13d, w2d)
+    out_acc = run_accurate(xd, lgd, w13d, w2d)
+    check_routing(get_workspace(DEV, T, 768, 1152, 8, 2), lg.float(), T)
+    check_outputs(f"h768_T{T}_{routing}", out_f32.cpu(), out_bf16.cpu(), ref, out_acc.cpu())
+
+
 @pytest.mark.parametrize("E,k", [(4, 1), (16, 4), (64, 8)])
 @pytest.mark.parametrize("T", [9, 70, 500])
 def test_layer_other_expert_counts(T, E, k):
