@@ -313,6 +313,21 @@ def test_layer_accurate_mode_with_bf16_output(T):
     assert float(((acc_bf16.float() - rounded).abs() - ulp).max()) <= slack
 
 
+@pytest.mark.parametrize("T", [8, 9, 16, 17, 63, 64, 191, 192, 193, 351, 352, 353, 447, 448, 449, 895, 896, 897,
+                               1023, 1024, 1025, 2047, 2048, 2049])
+def test_layer_at_every_kernel_switch(T):
+    """The batch sizes on both sides of every point where the layer changes kernels, K slices, sorted block,
+    routing front or the format of the partial results."""
+    announce(f"layer at a kernel switch, T={T}")
+    x, lg, w13, w2 = mid_inputs(T, "zipf", seed=11 * T)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out_f32, out_bf16 = run_both(xd, lgd, w13d, w2d)
+    out_acc = run_accurate(xd, lgd, w13d, w2d)
+    check_routing(get_workspace(DEV, T, MID["H"], MID["I"], 8, 2), lg.float(), T)
+    check_outputs(f"switch_T{T}", out_f32.cpu(), out_bf16.cpu(), ref, out_acc.cpu())
+
+
 @pytest.mark.parametrize("routing", ["normal", "one_expert"])
 @pytest.mark.parametrize("T", [40, 100, 300, 600, 1500])
 def test_layer_column_tiles_not_a_multiple_of_eight(T, routing):
