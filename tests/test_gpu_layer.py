@@ -313,6 +313,25 @@ def test_layer_accurate_mode_with_bf16_output(T):
     assert float(((acc_bf16.float() - rounded).abs() - ulp).max()) <= slack
 
 
+@pytest.mark.parametrize("routing", ["normal", "one_expert"])
+@pytest.mark.parametrize("I", [8192, 10240, 12288])
+@pytest.mark.parametrize("T", [96, 300])
+def test_layer_mid_kernel_many_column_tiles(T, I, routing):
+    """Wide intermediate sizes with H = 256: w13 launches of the 64- / 128-row kernel with two or three whole rounds
+    of 256-row weight tiles (I = 10240: plus a last round of 128-row tiles)."""
+    announce(f"layer H=256 I={I} T={T} {routing}")
+    x, lg, w13, w2 = O.make_inputs(T, 256, I, seed=T + I)
+    if routing == "one_expert":
+        lg = lg.float()
+        lg[:, 2] += 30.0
+        lg = lg.to(torch.bfloat16)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out_f32, out_bf16 = run_both(xd, lgd, w13d, w2d)
+    out_acc = run_accurate(xd, lgd, w13d, w2d)
+    check_outputs(f"wideI{I}_T{T}_{routing}", out_f32.cpu(), out_bf16.cpu(), ref, out_acc.cpu())
+
+
 @pytest.mark.parametrize("T", [8, 9, 16, 17, 63, 64, 191, 192, 193, 351, 352, 353, 447, 448, 449, 895, 896, 897,
                                1023, 1024, 1025, 2047, 2048, 2049])
 def test_layer_at_every_kernel_switch(T):
