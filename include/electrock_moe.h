@@ -262,9 +262,9 @@ typedef struct em_moe_layout {
     int64_t expert_ids_off, expert_ids_len;        /* [expert_ids_len] i32     */
     int64_t post_pad_off;                          /* [1] i32                  */
     int64_t seg_begin_off;                         /* [E+1] i32 padded segment starts */
-    int64_t act_off;                               /* [sorted_len, I] bf16     */
+    int64_t act_off;                               /* [sorted_len, I] bf16 (fp16 in accurate mode) */
     int64_t act_lo_off;                            /* [sorted_len, I] bf16, accurate mode of the generic kernels */
-    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 */
+    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 (fp16 above 448 tokens with a bf16 out) */
     int64_t total_bytes;
 } em_moe_layout;
 
