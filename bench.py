@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--accurate", action="store_true",
                     help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 instead of bf16 through the "
                          "w2 GEMM)")
+    ap.add_argument("--w2-f16", action="store_true",
+                    help="hand w2 over as float16 (converted once from the bf16 weights): accurate mode's arithmetic "
+                         "without the conversion inside the w2 kernels")
     ap.add_argument("--operands", choices=["gaussian", "zeros"], default="gaussian",
                     help="values of x and the expert weights.  'zeros' is a diagnostic: the matrix pipes then draw "
                          "little power and the same kernels run at the full shader clock, which separates the "
@@ -243,6 +246,9 @@ def main():
         print(json.dumps(vendor_gemm(torch, dev, args.tokens, min(args.steps, 30), min(args.warmup, 5))))
         return
     w13, w2 = make_weights(torch, dev)
+    if args.w2_f16:
+        w2 = w2.to(torch.float16)
+        LayerRunner.base_flags = _lib.FLAG_W2_F16
 
     T = args.tokens
     head = measure(torch, T, w13, w2, args.steps, args.warmup)
@@ -266,7 +272,7 @@ def main():
         for t in ((1, 8, 32, 64, 256) if args.shape == "8x7b" else (1, 64)):
             if t != T:
                 table.append(measure(torch, t, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2)))
-        if not args.accurate:  # the headline batch in accurate mode (fp16 activations)
+        if not args.accurate and not args.w2_f16:  # the headline batch in accurate mode (fp16 activations)
             from electrock_infer_amd import _lib
             LayerRunner.base_flags = _lib.FLAG_ACCURATE
             r = measure(torch, T, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2))
@@ -287,7 +293,8 @@ def main():
         "data": "synthetic" if args.operands == "gaussian" else "synthetic, all-zero x and weights (diagnostic)",
         "config": {"workload": f"Mixtral-{args.shape} MoE layer T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
                                f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
-                   "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate)},
+                   "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate or args.w2_f16),
+                   "w2_dtype": "f16" if args.w2_f16 else "bf16"},
         "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(torch, T, w13, w2),

@@ -18,6 +18,7 @@ NORM_LAYER, NORM_OP = 0, 1   # rounding points of layers/layernorm.py resp. of t
 FLAG_OUT_F32 = 1 << 0
 FLAG_ACCURATE = 1 << 1
 FLAG_GATE_F32_LOGITS = 1 << 2
+FLAG_W2_F16 = 1 << 3
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10

@@ -222,9 +222,10 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.w13 = static_cast<const uint16_t*>(w13);
     p.w2 = static_cast<const uint16_t*>(w2);
     p.act = reinterpret_cast<uint16_t*>(ws + L.act_off);
-    const bool accurate = (flags & EM_FLAG_ACCURATE) != 0;
+    const bool accurate = (flags & (EM_FLAG_ACCURATE | EM_FLAG_W2_F16)) != 0;
     p.act_lo = accurate ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
     p.act_f16 = 0;
+    p.w2_f16 = (flags & EM_FLAG_W2_F16) ? 1 : 0;
     p.y_f16 = 0;
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
@@ -247,6 +248,9 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.sorted_len = L.sorted_len;
     p.ksplit = static_cast<int>(L.ksplit);
 
+    // fp16 w2: only the tuned kernels have an fp16 w2 GEMM (checked before anything is launched)
+    if (p.w2_f16 && ((flags & EM_FLAG_FORCE_GENERIC) || !(T <= kStreamMaxT ? stream_supported(p) : tile_supported(p))))
+        return EM_ERR_UNSUPPORTED;
     const bool fused_front = !(flags & (EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN)) && norm == nullptr &&
                              gate_w == nullptr && route_align_supported(T, E, top_k);
     if (fused_front) {

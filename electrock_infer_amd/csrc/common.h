@@ -138,6 +138,7 @@ struct MoeProblem {
     uint16_t* act;            // [sorted_len, I] bf16, rows in sorted (padded) order
     uint16_t* act_lo;         // same shape: bf16(value - act) in the accurate mode of the generic kernels, else null
     int act_f16;              // act holds fp16 values (accurate mode of the tuned kernels; act_lo is null then)
+    int w2_f16;               // w2 holds fp16 values already: the fp16 w2 kernels skip their conversion
     int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
     int y_f16;                // y holds fp16 values instead (256-row kernel with a bf16 layer output)

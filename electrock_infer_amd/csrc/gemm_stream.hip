@@ -137,7 +137,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     bf[g] = *reinterpret_cast<const bf16x8_t*>(my + (g * 16 + r16) * kPitch + ks * 64 + kq * 16);
-                    if (F16) hf[g] = bf16x8_to_f16x8(bf[g]);
+                    if (F16) {
+                        if (p.w2_f16) __builtin_memcpy(&hf[g], &bf[g], 16);
+                        else hf[g] = bf16x8_to_f16x8(bf[g]);
+                    }
                 }
 #pragma unroll
                 for (int f = 0; f < kMaxF; ++f) {

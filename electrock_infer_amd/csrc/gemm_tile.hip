@@ -65,8 +65,9 @@ constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, se
 // STREAM: the weight rows are copied with the non-temporal hint.  Right when most experts fit one row tile
 // (every weight byte is then read by one workgroup only); wrong when several row tiles share them through L2.
 // F16 (w2 GEMM in accurate mode): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
-// into fp16 once, before its first MFMA, and the fp16 MFMA of the same shape and rate runs instead.
-template <int MODE, bool STREAM, bool F16>
+// into fp16 once, before its first MFMA, and the fp16 MFMA of the same shape and rate runs instead.  F16 = 1 converts
+// bf16 weights, F16 = 2 takes weights that are fp16 in memory (MoeProblem::w2_f16) as they come.
+template <int MODE, bool STREAM, int F16>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
                                                                int ntiles_n, int kslice) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         constexpr bool FULL = NMI == 4;
         constexpr int reads = decltype(reads_tag)::value;
         const int h = u & 1, k32 = u >> 1;
-        if (F16 && h == 0) convert_weights(k32);  // unit u is the first to use the weight fragments of this K half
+        if (F16 == 1 && h == 0) convert_weights(k32);  // unit u is the first to use the fragments of this K half
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (NMI ? (h * 4 + j < 2 * NMI) : (h * 4 + j < 2 * nmi)) {
@@ -514,12 +515,14 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev]) {
-        const void* kernels[6] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, false>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<1, true, false>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, false>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, false>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, true>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, true>)};
+        const void* kernels[8] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 0>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 1>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 1>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 2>),
+                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 2>)};
         for (const void* k : kernels) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
             if (e != hipSuccess) return static_cast<int>(e);
@@ -533,14 +536,17 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
         hipLaunchKernelGGL(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice);
     };
     if (mode == 1) {
-        if (stream_b) go(gemm_tile_kernel<1, true, false>, grid1, p.H);
-        else go(gemm_tile_kernel<1, false, false>, grid1, p.H);
+        if (stream_b) go(gemm_tile_kernel<1, true, 0>, grid1, p.H);
+        else go(gemm_tile_kernel<1, false, 0>, grid1, p.H);
+    } else if (p.act_f16 && p.w2_f16) {
+        if (stream_b) go(gemm_tile_kernel<2, true, 2>, grid2, p.I / p.ksplit);
+        else go(gemm_tile_kernel<2, false, 2>, grid2, p.I / p.ksplit);
     } else if (p.act_f16) {
-        if (stream_b) go(gemm_tile_kernel<2, true, true>, grid2, p.I / p.ksplit);
-        else go(gemm_tile_kernel<2, false, true>, grid2, p.I / p.ksplit);
+        if (stream_b) go(gemm_tile_kernel<2, true, 1>, grid2, p.I / p.ksplit);
+        else go(gemm_tile_kernel<2, false, 1>, grid2, p.I / p.ksplit);
     } else {
-        if (stream_b) go(gemm_tile_kernel<2, true, false>, grid2, p.I / p.ksplit);
-        else go(gemm_tile_kernel<2, false, false>, grid2, p.I / p.ksplit);
+        if (stream_b) go(gemm_tile_kernel<2, true, 0>, grid2, p.I / p.ksplit);
+        else go(gemm_tile_kernel<2, false, 0>, grid2, p.I / p.ksplit);
     }
     return launch_status();
 }

@@ -207,7 +207,10 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
     auto multiply_f16 = [&](int set) {
         f16x8_t hb[kCF];
 #pragma unroll
-        for (int g = 0; g < kCF; ++g) hb[g] = bf16x8_to_f16x8(fb[set][g]);
+        for (int g = 0; g < kCF; ++g) {
+            if (p.w2_f16) __builtin_memcpy(&hb[g], &fb[set][g], 16);
+            else hb[g] = bf16x8_to_f16x8(fb[set][g]);
+        }
 #pragma unroll
         for (int f = 0; f < kRF; ++f)
             if (f < nfr) {

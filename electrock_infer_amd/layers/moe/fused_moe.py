@@ -94,6 +94,16 @@ def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int) -> MoeWork
     return ws
 
 
+def _w2_flag(w2: torch.Tensor) -> int:
+    """w2 may be kept as float16 (converted once from the bfloat16 checkpoint, exactly for every weight of magnitude
+    2^-14 .. 65504): the layer then runs in accurate mode with no conversion in the w2 GEMM."""
+    if w2.dtype == torch.float16:
+        return _lib.FLAG_W2_F16
+    if w2.dtype != torch.bfloat16:
+        raise RuntimeError("the fused MoE path computes in bfloat16: w2 must be bfloat16 (or float16, see _w2_flag)")
+    return 0
+
+
 def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
                   gating_output: torch.Tensor, topk: int, renormalize: bool = True,
                   inplace: bool = False, activation: str = "silu",
@@ -107,7 +117,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     ``hidden_states`` and that tensor is returned, as in the reference.
     ``out_dtype=torch.float32`` returns the un-rounded fp32 result instead
     (not available together with ``inplace``).  ``accurate=True`` keeps the
-    SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM.
+    SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM; a float16
+    ``w2`` does the same without the conversion of the weights inside the kernel.
     """
     if activation != "silu":
         raise NotImplementedError(f"Activation {activation} not supported.")
@@ -119,8 +130,9 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         raise RuntimeError("weight shapes do not match hidden_states")
     if gating_output.shape[0] != T or gating_output.shape[1] != E:
         raise RuntimeError("gating_output must be [num_tokens, num_experts]")
-    if not (hidden_states.dtype == w1.dtype == w2.dtype == torch.bfloat16):
+    if not (hidden_states.dtype == w1.dtype == torch.bfloat16):
         raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, w1 and w2 must be bfloat16")
+    flags |= _w2_flag(w2)
     want_f32 = out_dtype == torch.float32
     if accurate:
         flags |= _lib.FLAG_ACCURATE
@@ -185,8 +197,9 @@ def fused_experts_gated(hidden_states: torch.Tensor, gate_weight: torch.Tensor, 
         raise RuntimeError("weight shapes do not match hidden_states")
     if tuple(gate_weight.shape) != (E, H):
         raise RuntimeError("gate_weight must be [num_experts, hidden_size]")
-    if not (hidden_states.dtype == gate_weight.dtype == w1.dtype == w2.dtype == torch.bfloat16):
+    if not (hidden_states.dtype == gate_weight.dtype == w1.dtype == torch.bfloat16):
         raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, gate_weight, w1 and w2 must be bfloat16")
+    flags |= _w2_flag(w2)
     want_f32 = out_dtype == torch.float32
     if accurate:
         flags |= _lib.FLAG_ACCURATE
@@ -270,8 +283,9 @@ def fused_experts_normed(hidden_states: torch.Tensor, residual: Optional[torch.T
     I = two_i // 2
     if Hw != H or tuple(w2.shape) != (E, H, I) or two_i != 2 * I or tuple(gate_weight.shape) != (E, H):
         raise RuntimeError("weight shapes do not match hidden_states")
-    if not (w1.dtype == w2.dtype == torch.bfloat16):
+    if w1.dtype != torch.bfloat16:
         raise RuntimeError("the fused MoE path computes in bfloat16: w1 and w2 must be bfloat16")
+    flags |= _w2_flag(w2)
     if accurate:
         flags |= _lib.FLAG_ACCURATE
     if not bf16_logits:

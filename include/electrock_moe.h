@@ -47,6 +47,7 @@ extern "C" {
 #define EM_FLAG_ACCURATE       (1u << 1)  /* SiLU*mul activations kept beyond one bf16       */
 #define EM_FLAG_GATE_F32_LOGITS (1u << 2) /* em_moe_forward_gated: route on the fp32 logits,   */
                                           /* not on their bf16 rounding                        */
+#define EM_FLAG_W2_F16         (1u << 3)  /* `w2` holds fp16 values; implies EM_FLAG_ACCURATE */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
 #define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
 #define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
@@ -230,6 +231,11 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  * (value, rounding residual) and the residual is multiplied in a second pass over
  * w2.  Both forms meet max-abs 2e-2 / mean relative 1e-3 against the fp32 definition
  * with EM_FLAG_OUT_F32.
+ * EM_FLAG_W2_F16: the caller keeps w2 as fp16 (converted once, e.g. when the weights
+ * are loaded: exact for every bf16 weight of magnitude 2^-14 .. 65504).  The layer then
+ * runs in accurate mode without the conversion: within 1-2 % of the default mode's time
+ * at every batch size.  Only shapes the tuned kernels take; others return
+ * EM_ERR_UNSUPPORTED.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.

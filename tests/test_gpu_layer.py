@@ -297,6 +297,42 @@ def test_layer_router_and_sort_in_one_launch(T, dtype):
     check_routing(get_workspace(DEV, T, 256, 512, 8, 2), lg.float(), T)
 
 
+@pytest.mark.parametrize("T", [1, 7, 33, 64, 200, 400, 777, 2100])
+def test_layer_with_float16_w2(T):
+    """w2 handed over as float16 (converted once from bf16: exact in this range) runs the accurate mode's arithmetic
+    without the conversion inside the w2 kernels: the same results as accurate mode on the bf16 weights up to the
+    rounding of the few weights below 2^-14 in magnitude (fp16 subnormals: torch rounds them to nearest, the kernels'
+    conversion towards zero), and the stated target against the oracle.  The generic kernels refuse float16 w2."""
+    announce(f"layer with float16 w2, T={T}")
+    x, lg, w13, w2 = mid_inputs(T, "zipf", seed=5 * T)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    w2h = w2d.to(torch.float16)
+    out = fused_experts(xd, w13d, w2h, lgd, 2, renormalize=True, out_dtype=torch.float32)
+    st = error_stats(out.cpu(), ref)
+    record(f"w2f16_T{T}", f32=st)
+    assert st["max_abs"] <= TARGET_MAX_ABS and st["mean_rel"] <= TARGET_MEAN_REL, st
+    acc = run_accurate(xd, lgd, w13d, w2d)
+    assert float((out - acc).abs().max()) <= 1e-6 * float(ref.abs().max())
+    with pytest.raises(RuntimeError):
+        fused_experts(xd, w13d, w2h, lgd, 2, flags=_lib.FLAG_FORCE_GENERIC)
+
+
+def test_fusedmoe_module_with_float16_w2():
+    announce("FusedMoE module, w2_dtype=float16")
+    x, lg, w13, w2 = O.make_inputs(70, MID["H"], MID["I"], seed=70)
+    layer = FusedMoE(num_experts=8, top_k=2, hidden_size=MID["H"], intermediate_size=MID["I"], tp_size=1,
+                     params_dtype=torch.bfloat16, w2_dtype=torch.float16).to(DEV)
+    assert layer.w2_weight.dtype == torch.float16 and layer.w13_weight.dtype == torch.bfloat16
+    for e in range(8):   # the reference loader's calls (utils/loader.py:36-49): the copy converts w2
+        layer.weight_loader(layer.w13_weight, w13[e, :MID["I"]].to(DEV), "w1", e)
+        layer.weight_loader(layer.w13_weight, w13[e, MID["I"]:].to(DEV), "w3", e)
+        layer.weight_loader(layer.w2_weight, w2[e].to(DEV), "w2", e)
+    xd = x.to(DEV)
+    expect = fused_experts(xd.clone(), w13.to(DEV), w2.to(DEV), lg.to(DEV), 2, accurate=True)
+    assert torch.equal(layer(xd, lg.to(DEV)), expect)
+
+
 @pytest.mark.parametrize("T", [7, 64, 300, 777])
 def test_layer_accurate_mode_with_bf16_output(T):
     """Accurate mode is asserted against the stated target with an fp32 output everywhere else; with the default bf16
