@@ -134,8 +134,8 @@ int launch_rms_norm(const void* x_in, const void* res_in, const void* weight, vo
 struct MoeProblem {
     const uint16_t* x;        // [T, H] bf16
     const uint16_t* w13;      // [E, 2I, H] bf16
-    const uint16_t* w2;       // [E, H, I] bf16
-    uint16_t* act;            // [sorted_len, I] bf16, rows in sorted (padded) order
+    const uint16_t* w2;       // [E, H, I] bf16 (fp16 when w2_f16)
+    uint16_t* act;            // [sorted_len, I] bf16 (fp16 when act_f16), rows in sorted (padded) order
     uint16_t* act_lo;         // same shape: bf16(value - act) in the accurate mode of the generic kernels, else null
     int act_f16;              // act holds fp16 values (accurate mode of the tuned kernels; act_lo is null then)
     int w2_f16;               // w2 holds fp16 values already: the fp16 w2 kernels skip their conversion

@@ -15,7 +15,7 @@
 //   * the four partial accumulators meet once, at the end, in LDS.
 //
 //   MODE 1  64 rows = 32 gate rows j and the 32 up rows I + j of w13[e]; epilogue
-//           act[p, j] = bf16(silu(g) * u) with g, u still in fp32
+//           act[p, j] = silu(g) * u with g, u still in fp32, rounded once (bf16; fp16 in accurate mode)
 //           (reference: Triton GEMM #1 + _C.silu_and_mul, fused_moe.py:250-272)
 //   MODE 2  64 rows n of w2[e], K slice z of I; epilogue y[z, slot, n] = partial sum
 //           (reference: Triton GEMM #2, fused_moe.py:282-287)
@@ -41,7 +41,8 @@ __device__ __forceinline__ u32x4_t ld16_stream(const uint16_t* p) {
 }
 
 // F16 (accurate mode, MODE 2 only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are turned
-// into fp16 between the LDS tile and the MFMA, which costs this HBM-bound kernel nothing.
+// into fp16 between the LDS tile and the MFMA (not when they are fp16 in memory, MoeProblem::w2_f16), which costs
+// this HBM-bound kernel nothing.
 template <int MODE, bool F16>
 __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem p,
                                                                      const int32_t* __restrict__ seg_begin,

@@ -67,7 +67,8 @@ __device__ __forceinline__ void wait_stages(int stages) {
 // One tile: `block` is the workgroup's index among those of its tile width, `col0` the first weight row
 // (MODE 1: first gate row) of the range that this width covers, `ntiles_n` the tiles across that range.
 // F16 (w2 GEMM only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are converted on their
-// way from LDS to the MFMA, which costs this HBM-bound kernel nothing.
+// way from LDS to the MFMA (not when they are fp16 in memory, MoeProblem::w2_f16), which costs this HBM-bound kernel
+// nothing.
 template <int MODE, int MI, int NT, bool F16>
 __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __restrict__ seg_begin, int block, int col0,
                                           int ntiles_n, int kslice, uint8_t* smem) {
