@@ -188,6 +188,21 @@ def test_layer_8x7b_prefill(mixtral_8x7b, logits):
     assert torch.allclose(out_p, out_f32[perm], rtol=0, atol=1e-5)
 
 
+def test_layer_8x7b_float16_w2(mixtral_8x7b):
+    """w2 handed over as float16 at the full 8x7B shape (decode, mid-size and prefill kernels): the stated target
+    against the oracle on sampled tokens."""
+    m = mixtral_8x7b
+    w2h = m["w2"].to(torch.float16)
+    for T in (1, 64, 256, 8192):
+        announce(f"layer 8x7B float16 w2 T={T}")
+        x, lg = m["x"][:T].contiguous(), m["lg"][:T].contiguous()
+        out = fused_experts(x, m["w13"], w2h, lg, 2, out_dtype=torch.float32)
+        rows = list(range(T)) if T <= 64 else list(range(0, T, T // 64))
+        st = error_stats(out[rows].cpu(), oracle_rows(x, lg, m["w13_cpu"], m["w2_cpu"], rows))
+        record(f"8x7b_w2f16_T{T}", f32=st)
+        assert st["max_abs"] <= TARGET_MAX_ABS and st["mean_rel"] <= TARGET_MEAN_REL, st
+
+
 def test_layer_8x22b_shape():
     """Configuration 5: H=6144, I=16384; T in {1, 64} in full, T=4096 on sampled tokens."""
     announce("building 8x22B-shaped weights")
