@@ -47,9 +47,9 @@ def record(case: str, **stats):
     print(f"[layer-error] {case} {stats}", flush=True)
 
 
-def check_routing(ws, lg_cpu_f32, T, E=8, k=2):
+def check_routing(ws, lg_cpu_f32, T, E=8, k=2, renormalize=True):
     """Bit-exact comparison of everything the router and the sort left in the workspace."""
-    ow, oids = O.topk_softmax(lg_cpu_f32.numpy(), k, True)
+    ow, oids = O.topk_softmax(lg_cpu_f32.numpy(), k, renormalize)
     ids = ws.topk_ids().cpu().numpy()
     assert np.array_equal(ids, oids)
     np.testing.assert_allclose(ws.topk_weights().cpu().numpy(), ow, rtol=2e-6, atol=1e-9)
@@ -461,6 +461,40 @@ def test_layer_mid_shape_decode_cases(T, routing):
     check_outputs(f"mid_dec_T{T}_{routing}", out_f32.cpu(), out_bf16.cpu(), ref, out_acc.cpu())
     gen_f32, gen_bf16 = run_both(xd, lgd, w13d, w2d, flags=_lib.FLAG_FORCE_GENERIC)
     check_outputs(f"mid_dec_T{T}_{routing}_generic", gen_f32.cpu(), gen_bf16.cpu(), ref)
+
+
+def _drawn_case(seed):
+    """Shape, batch and routing of one drawn case (a fixed function of the seed)."""
+    rng = np.random.default_rng(1000 + seed)
+    H = int(rng.choice([64, 136, 256, 320, 512, 768, 1024, 1280, 2048]))
+    I = int(rng.choice([64, 200, 256, 384, 512, 640, 1024, 1152, 1536, 2048, 3584]))
+    E, k = [(8, 2), (8, 2), (8, 2), (8, 1), (4, 2), (16, 2), (2, 2), (32, 3), (64, 6)][int(rng.integers(9))]
+    T = int(rng.choice([1, 2, 5, 8, 9, 16, 17, 31, 48, 64, 65, 100, 129, 192, 193, 250, 352, 353, 449, 600, 897, 1300, 2049, 2100]))
+    routing = ["normal", "zipf", "two_experts"][int(rng.integers(3))]
+    logits_dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(3))]
+    return H, I, E, k, T, routing, logits_dtype, bool(rng.integers(2))
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_layer_drawn_shapes(seed):
+    """Shapes, expert counts, batch sizes, routing skews, logit types and the renormalise switch drawn together: whatever
+    kernels the library picks for the combination, routing bit-exact and outputs within the tolerances."""
+    H, I, E, k, T, routing, logits_dtype, renorm = _drawn_case(seed)
+    announce(f"drawn case {seed}: H={H} I={I} E={E} top-{k} T={T} {routing} logits={logits_dtype} renormalize={renorm}")
+    x, lg, w13, w2 = O.make_inputs(T, H, I, E=E, seed=seed, logits=routing, logits_dtype=logits_dtype)
+    ref = O.moe_layer_fp32(x, lg, w13, w2, topk=k, renormalize=renorm)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out = fused_experts(xd, w13d, w2d, lgd, k, renormalize=renorm, out_dtype=torch.float32)
+    check_routing(get_workspace(DEV, T, H, I, E, k), lg.float(), T, E=E, k=k, renormalize=renorm)
+    st = error_stats(out.cpu(), ref)
+    record(f"drawn_{seed}", f32=st)
+    assert st["mean_rel"] <= TOL_MEAN_REL_F32 and st["max_abs"] <= TOL_MAX_ABS_F32 * float(ref.abs().max()), st
+    acc = fused_experts(xd, w13d, w2d, lgd, k, renormalize=renorm, out_dtype=torch.float32, accurate=True)
+    sa = error_stats(acc.cpu(), ref)
+    assert sa["max_abs"] <= TARGET_MAX_ABS and sa["mean_rel"] <= TARGET_MEAN_REL, sa
+    out_b = fused_experts(xd, w13d, w2d, lgd, k, renormalize=renorm)
+    sb = error_stats(out_b.float().cpu(), ref)
+    assert sb["mean_rel"] <= TOL_MEAN_REL_BF16, sb
 
 
 def test_layer_shape_only_the_generic_kernel_supports():
