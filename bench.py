@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the Mixtral-8x7B MoE layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T] [--no-cpu] [--no-table]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T] [--shape 8x7b|8x22b] [--accurate | --w2-f16]
+                    [--no-cpu] [--no-table]
 
 A "step" is one call of the layer (router, expert sort, w13 GEMM + SiLU*mul,
 w2 GEMM, top-k combine) on one batch of T tokens resident in HBM.  The headline
