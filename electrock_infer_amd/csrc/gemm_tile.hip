@@ -42,6 +42,8 @@
 //              takes an eighth of the column tiles of every expert and walks them expert by
 //              expert, column by column, row tile fastest, so that the 32 CUs of an XCD share
 //              weight and token tiles through their own L2 and weights leave HBM once.
+#include <atomic>
+
 #include "common.h"
 #include "lds_copy.h"
 #include <type_traits>
@@ -511,10 +513,10 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     constexpr int lds_bytes = kLdsBytes;
     // Opt in to more than 64 KB of dynamic LDS once per device.  The flags only cache an
     // idempotent runtime call; a race between threads at worst repeats it.
-    static bool attr_set[64] = {};
+    static std::atomic<bool> attr_set[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (!attr_set[dev]) {
+    if (!attr_set[dev].load(std::memory_order_acquire)) {
         const void* kernels[8] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0>),
                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0>),
                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0>),
@@ -527,7 +529,7 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
             if (e != hipSuccess) return static_cast<int>(e);
         }
-        attr_set[dev] = true;
+        attr_set[dev].store(true, std::memory_order_release);
     }
     // one row tile per expert on average up to 7/8 full: weights are read once -> streaming copies
     const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * 7;

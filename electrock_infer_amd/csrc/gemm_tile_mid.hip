@@ -23,6 +23,8 @@
 //   K order    every tile starts at its own K offset and wraps around (see `rot` below)
 //   the rest   LDS swizzle, gate/up pairing in one lane, XCD-aware tile order, split-K for w2
 //              and the LDS-turned epilogues are those of the 256-row kernel.
+#include <atomic>
+
 #include "common.h"
 #include "lds_copy.h"
 
@@ -352,14 +354,14 @@ int launch_mid(const MoeProblem& p, const int32_t* seg_begin, hipStream_t s) {
     const int wide_blocks = static_cast<int>(round_up(max_mtiles * ntn_wide, kXcds));
     const unsigned grid = static_cast<unsigned>(wide_blocks + round_up(max_mtiles * ntn_narrow, kXcds));
     if (grid == 0) return 0;
-    static bool attr_set[64] = {};  // caches an idempotent runtime call per device
+    static std::atomic<bool> attr_set[64];  // caches an idempotent runtime call per device
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (!attr_set[dev]) {
+    if (!attr_set[dev].load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tile_mid_kernel<MODE, MI, F16>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
         if (e != hipSuccess) return static_cast<int>(e);
-        attr_set[dev] = true;
+        attr_set[dev].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((gemm_tile_mid_kernel<MODE, MI, F16>), dim3(grid, static_cast<unsigned>(slices)), dim3(kThreads),
                        kLdsBytes, s, p, seg_begin, wide_blocks, ntn_wide, col0n, ntn_narrow,

@@ -84,6 +84,9 @@ _workspaces: Dict[tuple, MoeWorkspace] = {}
 
 
 def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int) -> MoeWorkspace:
+    """The cached workspace of a device.  Calls on one device share it: they have to be ordered on one stream (as the
+    layers of a model are); a caller that runs layer calls on several streams at once passes each its own
+    ``MoeWorkspace`` through the ``workspace`` argument of the entry points."""
     key = (torch.device(device).index, T, H, I, E, top_k)
     ws = _workspaces.get(key)
     if ws is None:
