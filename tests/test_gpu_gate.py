@@ -42,7 +42,7 @@ def test_gate_topk_matches_oracle(T, H, E, bf16_logits):
         sum_abs = np.abs(x.float().cpu().numpy()).astype(np.float64) @ np.abs(gw.float().cpu().numpy()).astype(np.float64).T
         err = np.abs(got - want)
         assert (err <= bf16_ulp(want) * (1.0 + 1e-6) + 4 * 2.0 ** -24 * sum_abs).all()
-        assert (err > 0).mean() < 2e-3
+        assert (err > 0).sum() <= max(2, 2e-3 * err.size)   # (a small batch may hold one such logit)
     else:
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
     # the selection must be the oracle's selection on the logits the kernel itself produced (bit-exact ids),
