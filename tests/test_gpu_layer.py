@@ -348,6 +348,38 @@ def test_fusedmoe_module_with_float16_w2():
     assert torch.equal(layer(xd, lg.to(DEV)), expect)
 
 
+@pytest.mark.parametrize("T", [5, 100, 600])
+def test_accurate_mode_clamps_activations_at_the_fp16_range(T):
+    """The documented difference between the two modes: fp16 activations saturate at +-65504, bf16 ones do not.
+    Inputs whose SiLU*mul values pass that bound: the default mode follows the fp32 definition, accurate mode the
+    definition with the activations clamped."""
+    announce(f"activation range, T={T}")
+    x, lg, w13, w2 = mid_inputs(T, "normal", seed=900 + T)
+    x, w13 = (x.float() * 30).to(torch.bfloat16), (w13.float() * 50).to(torch.bfloat16)
+    I = MID["I"]
+    w, ids = O.topk_softmax(lg.float().numpy(), 2, True)
+    ref = torch.zeros(T, MID["H"])
+    ref_clamped = torch.zeros(T, MID["H"])
+    over = 0
+    for t in range(T):
+        for j in range(2):
+            e = int(ids[t, j])
+            h = w13[e].float() @ x[t].float()
+            act = torch.nn.functional.silu(h[:I]) * h[I:]
+            over += int((act.abs() > 65504).sum())
+            ref[t] += float(w[t, j]) * (w2[e].float() @ act)
+            ref_clamped[t] += float(w[t, j]) * (w2[e].float() @ act.clamp(-65504, 65504))
+    assert over > 10 * T                                   # the bound really is passed, many times per token
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out = fused_experts(xd, w13d, w2d, lgd, 2, out_dtype=torch.float32).cpu()
+    acc = fused_experts(xd, w13d, w2d, lgd, 2, out_dtype=torch.float32, accurate=True).cpu()
+    assert torch.isfinite(out).all() and torch.isfinite(acc).all()
+    scale = float(ref.abs().max())
+    assert float((out - ref).abs().max()) <= TOL_MAX_ABS_F32 * scale
+    assert float((acc - ref_clamped).abs().max()) <= 1e-3 * scale
+    assert float((ref - ref_clamped).abs().max()) > 20e-3 * scale      # the two definitions are well apart here
+
+
 @pytest.mark.parametrize("T", [7, 64, 300, 777])
 def test_layer_accurate_mode_with_bf16_output(T):
     """Accurate mode is asserted against the stated target with an fp32 output everywhere else; with the default bf16
