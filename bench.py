@@ -46,6 +46,8 @@ def parse_args():
     ap.add_argument("--accurate", action="store_true",
                     help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 instead of bf16 through the "
                          "w2 GEMM)")
+    ap.add_argument("--wide-range", action="store_true",
+                    help="EM_FLAG_WIDE_RANGE: float32 partial sums of the w2 GEMM at every batch size")
     ap.add_argument("--w2-f16", action="store_true",
                     help="hand w2 over as float16 (converted once from the bf16 weights): accurate mode's arithmetic "
                          "without the conversion inside the w2 kernels")
@@ -250,6 +252,8 @@ def main():
     if args.w2_f16:
         w2 = w2.to(torch.float16)
         LayerRunner.base_flags = _lib.FLAG_W2_F16
+    if args.wide_range:
+        LayerRunner.base_flags |= _lib.FLAG_WIDE_RANGE
 
     T = args.tokens
     head = measure(torch, T, w13, w2, args.steps, args.warmup)

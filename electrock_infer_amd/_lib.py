@@ -19,6 +19,7 @@ FLAG_OUT_F32 = 1 << 0
 FLAG_ACCURATE = 1 << 1
 FLAG_GATE_F32_LOGITS = 1 << 2
 FLAG_W2_F16 = 1 << 3
+FLAG_WIDE_RANGE = 1 << 4
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10

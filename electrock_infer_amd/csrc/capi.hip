@@ -290,7 +290,8 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     // Where the output is bf16, the partial results of the 256-row w2 kernel are fp16 (their rounding, 2^-12, is far
     // below the output's, 2^-9): half the bytes written by the kernel's epilogues, which all fall into the same
     // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer).
-    if (use_tile && T > kTile128W2MaxT && !(flags & EM_FLAG_OUT_F32)) p.y_f16 = 1;
+    // fp16 saturates at 65504: EM_FLAG_WIDE_RANGE keeps the partial results float32 for callers whose values may pass it.
+    if (use_tile && T > kTile128W2MaxT && !(flags & (EM_FLAG_OUT_F32 | EM_FLAG_WIDE_RANGE))) p.y_f16 = 1;
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
         if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);

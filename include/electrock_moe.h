@@ -48,6 +48,8 @@ extern "C" {
 #define EM_FLAG_GATE_F32_LOGITS (1u << 2) /* em_moe_forward_gated: route on the fp32 logits,   */
                                           /* not on their bf16 rounding                        */
 #define EM_FLAG_W2_F16         (1u << 3)  /* `w2` holds fp16 values; implies EM_FLAG_ACCURATE */
+#define EM_FLAG_WIDE_RANGE     (1u << 4)  /* bf16 output: w2 partial sums stay float32 at   */
+                                          /* every batch size (see em_moe_forward)          */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
 #define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
 #define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
@@ -236,6 +238,10 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  * runs in accurate mode without the conversion: within 1-2 % of the default mode's time
  * at every batch size.  Only shapes the tuned kernels take; others return
  * EM_ERR_UNSUPPORTED.
+ * Range: above 448 tokens with a bf16 output the partial sums of the w2 GEMM (one per
+ * routed slot and K slice, before the routing weight) pass through fp16 and saturate at
+ * +-65504, where the reference's bf16 pipeline does not.  EM_FLAG_WIDE_RANGE keeps them
+ * float32 (T=8192: +1-2 % in time); a float32 output always does.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.

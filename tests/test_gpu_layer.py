@@ -380,6 +380,25 @@ def test_accurate_mode_clamps_activations_at_the_fp16_range(T):
     assert float((ref - ref_clamped).abs().max()) > 20e-3 * scale      # the two definitions are well apart here
 
 
+def test_wide_range_flag_keeps_partial_sums_in_float32():
+    """Above 448 tokens a bf16 output takes the partial sums of the w2 GEMM through fp16, which saturates at 65504;
+    FLAG_WIDE_RANGE keeps them float32, and the layer then follows the definition at any magnitude bf16 holds."""
+    T = 600
+    announce(f"output range, T={T}")
+    x, lg, w13, w2 = mid_inputs(T, "normal", seed=31)
+    x, w2 = (x.float() * 300).to(torch.bfloat16), (w2.float() * 300).to(torch.bfloat16)
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    scale = float(ref.abs().max())
+    assert scale > 4 * 65504
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    wide = fused_experts(xd, w13d, w2d, lgd, 2, flags=_lib.FLAG_WIDE_RANGE).float().cpu()
+    assert float((wide - ref).abs().max()) <= 2.0 ** -7 * scale
+    narrow = fused_experts(xd, w13d, w2d, lgd, 2).float().cpu()
+    assert torch.isfinite(narrow).all()
+    assert float(narrow.abs().max()) <= 4 * 65504 * 1.01        # two slots x two K slices, each saturated at most
+    assert float((narrow - ref).abs().max()) > 0.1 * scale
+
+
 @pytest.mark.parametrize("T", [7, 64, 300, 777])
 def test_layer_accurate_mode_with_bf16_output(T):
     """Accurate mode is asserted against the stated target with an fp32 output everywhere else; with the default bf16
