@@ -5,8 +5,8 @@
  * Every entry point takes raw DEVICE pointers, plain sizes and a HIP stream
  * (passed as void* so that this header needs no HIP include), launches
  * asynchronously on that stream, never allocates, frees or retains memory and
- * keeps no mutable global state.  The caller guarantees that the device owning
- * the pointers is current.
+ * keeps no state between calls (but a per-device note that a kernel attribute has
+ * been set).  The caller guarantees that the device owning the pointers is current.
  *
  * Return value of every function returning int:
  *     0   success (work is queued on `stream`)
@@ -221,7 +221,7 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  *   router_logits [T, E]      logits_dtype in {F32, BF16, F16}
  *   w13           [E, 2I, H]  bf16, rows [0,I) = gate (w1), rows [I,2I) = up (w3)
  *                             (mixtral_moe.py:64-70,137-143)
- *   w2            [E, H, I]   bf16 (mixtral_moe.py:75-79)
+ *   w2            [E, H, I]   bf16 (mixtral_moe.py:75-79); fp16 with EM_FLAG_W2_F16
  *   out           [T, H]      bf16 (float32 with EM_FLAG_OUT_F32); may alias x
  *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k), 256-byte aligned
  * EM_FLAG_ACCURATE takes the one rounding to bf16 that the MFMA of the w2 GEMM
