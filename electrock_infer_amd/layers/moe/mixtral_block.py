@@ -40,18 +40,20 @@ class MixtralMoE(nn.Module):
     """``forward(hidden_states)`` = ``experts(hidden_states, gate(hidden_states))`` of the reference
     (models/mixtral.py:53-63), with the gate computed inside the router's launch.  ``bf16_logits=True``
     (default) rounds the logits to bf16 before the selection as the reference's bf16 gate does; ``accurate=True``
-    keeps the SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM."""
+    keeps the SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM; ``w2_dtype=torch.float16`` keeps
+    ``experts.w2_weight`` as float16 (the loader's copy converts), which implies it at no cost in time."""
 
     def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int,
                  params_dtype: Optional[torch.dtype] = None, tp_size: Optional[int] = None, prefix: str = "",
-                 bf16_logits: bool = True, accurate: bool = False):
+                 bf16_logits: bool = True, accurate: bool = False, w2_dtype: Optional[torch.dtype] = None):
         super().__init__()
         self.hidden_size = hidden_size
         self.bf16_logits = bf16_logits
         self.gate = ReplicatedLinear(hidden_size, num_experts, bias=False, params_dtype=params_dtype)
         self.experts = FusedMoE(num_experts=num_experts, top_k=top_k, hidden_size=hidden_size,
                                 intermediate_size=intermediate_size, params_dtype=params_dtype,
-                                reduce_results=True, renormalize=True, tp_size=tp_size, accurate=accurate)
+                                reduce_results=True, renormalize=True, tp_size=tp_size, accurate=accurate,
+                                w2_dtype=w2_dtype)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         orig_shape = hidden_states.shape

@@ -62,6 +62,22 @@ def test_load_model_stacks_expert_weights(tmp_path):
         assert torch.equal(layer.post_attention_layernorm.weight.to(torch.bfloat16), t[pre + "post_attention_layernorm.weight"])
 
 
+def test_load_model_converts_w2_for_a_float16_w2_parameter(tmp_path):
+    """w2_dtype=float16: the parameter is float16 and the loader's copy converts the checkpoint's bfloat16 tensors
+    (exactly: these values lie inside the fp16 range)."""
+    E, H, I = 2, 16, 24
+    t = _checkpoint(tmp_path, E, H, I, layers=1, extra=False)
+    m = _Model(E, H, I, layers=1)
+    m.model.layers[0].block_sparse_moe = MixtralMoE(E, 2, H, I, params_dtype=torch.bfloat16, tp_size=1,
+                                                    w2_dtype=torch.float16)
+    load_model(m, str(tmp_path), strict=True)
+    ex = m.model.layers[0].block_sparse_moe.experts
+    assert ex.w2_weight.dtype == torch.float16 and ex.w13_weight.dtype == torch.bfloat16
+    for e in range(E):
+        src = t[f"model.layers.0.block_sparse_moe.experts.{e}.w2.weight"]
+        assert torch.equal(ex.w2_weight[e].float(), src.float())
+
+
 def test_load_model_strict_raises_on_unknown_tensor(tmp_path):
     _checkpoint(tmp_path, 2, 8, 8, layers=1)
     with pytest.raises(AttributeError):
