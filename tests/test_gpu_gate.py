@@ -111,3 +111,24 @@ def test_mixtral_block_module():
     ref = O.moe_layer_fp32(x0.view(-1, H).cpu(), torch.from_numpy(logits), blk.experts.w13_weight.cpu(), blk.experts.w2_weight.cpu())
     st = error_stats(y.view(-1, H), ref)
     assert st["mean_rel"] <= 6e-3, st
+
+
+def test_mixtral_block_module_with_float16_w2():
+    """w2_dtype=float16 on the block: the same call as accurate mode on the bf16 weights, without the conversion."""
+    from electrock_infer_amd import MixtralMoE
+    from electrock_infer_amd.layers.moe.fused_moe import fused_experts_gated
+    announce("MixtralMoE module, float16 w2")
+    T, H, I, E = 200, 256, 512, 8
+    g = torch.Generator().manual_seed(5)
+    blk = MixtralMoE(E, 2, H, I, params_dtype=torch.bfloat16, w2_dtype=torch.float16).to(DEV)
+    assert blk.experts.w2_weight.dtype == torch.float16
+    blk.gate.weight.data.copy_((torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16))
+    blk.experts.w13_weight.data.copy_((torch.randn(E, 2 * I, H, generator=g) * 0.02).to(torch.bfloat16))
+    w2 = (torch.randn(E, H, I, generator=g) * 0.02).to(torch.bfloat16).to(DEV)
+    for e in range(E):
+        blk.experts.weight_loader(blk.experts.w2_weight, w2[e], "w2", e)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(DEV)
+    want = fused_experts_gated(x.clone(), blk.gate.weight, blk.experts.w13_weight, w2, topk=2, renormalize=True,
+                               accurate=True)
+    got = blk(x.clone())
+    assert float((got.float() - want.float()).abs().max()) <= 2.0 ** -8 * float(want.float().abs().max())
