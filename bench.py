@@ -14,6 +14,7 @@ One JSON line is printed.  Besides the contract fields it carries
                 events on the stream it is launched on, against 8 TB/s of HBM
   cpu_baseline  the reference-style torch CPU expert loop (oracle port) timed on
                 the host cores on the same workload
+  latency_us    p10 / p50 / p90 of single layer calls, each between its own pair of events
   table         layer latency / HBM GB/s / MFMA TFLOP/s for the other batch sizes
                 of the decode list, the headline batch in accurate mode and the
                 T=8192 prefill cases
@@ -46,6 +47,9 @@ def parse_args():
     ap.add_argument("--accurate", action="store_true",
                     help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 instead of bf16 through the "
                          "w2 GEMM)")
+    ap.add_argument("--weight-sets", type=int, default=1,
+                    help="cycle the calls through N independently drawn sets of expert weights (N x 2.8 GB), so that no "
+                         "call finds the weights of the one before in a cache")
     ap.add_argument("--wide-range", action="store_true",
                     help="EM_FLAG_WIDE_RANGE: float32 partial sums of the w2 GEMM at every batch size")
     ap.add_argument("--w2-f16", action="store_true",
@@ -67,8 +71,8 @@ def parse_args():
 OPERANDS = "gaussian"
 
 
-def make_weights(torch, dev):
-    g = torch.Generator(device=dev).manual_seed(0)
+def make_weights(torch, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
     if OPERANDS == "zeros":
         return (torch.zeros(E, 2 * I, H, device=dev, dtype=torch.bfloat16),
                 torch.zeros(E, H, I, device=dev, dtype=torch.bfloat16))
@@ -99,6 +103,7 @@ class LayerRunner:
     """Calls em_moe_forward through the C ABI with pre-allocated buffers."""
 
     base_flags = 0
+    extra_weight_sets = []      # [(w13, w2), ...] cycled through together with the set given to the constructor
 
     def __init__(self, torch, T, w13, w2, x, lg):
         import ctypes
@@ -106,13 +111,20 @@ class LayerRunner:
         from electrock_infer_amd.layers.moe.fused_moe import MoeWorkspace
         self.torch, self._lib, self.ctypes = torch, _lib, ctypes
         self.T, self.w13, self.w2, self.x, self.lg = T, w13, w2, x, lg
+        self.more_sets, self.calls = LayerRunner.extra_weight_sets, 0
         self.ws = MoeWorkspace(x.device, T, H, I, E, TOPK)
         self.out = torch.empty_like(x)
         self.lib = _lib.load()
 
     def __call__(self, flags=0):
+        w13, w2 = self.w13, self.w2
+        if self.more_sets:
+            k = self.calls % (len(self.more_sets) + 1)
+            self.calls += 1
+            if k:
+                w13, w2 = self.more_sets[k - 1]
         code = self.lib.em_moe_forward(
-            self.x.data_ptr(), self.lg.data_ptr(), self._lib.DTYPE_BF16, self.w13.data_ptr(), self.w2.data_ptr(),
+            self.x.data_ptr(), self.lg.data_ptr(), self._lib.DTYPE_BF16, w13.data_ptr(), w2.data_ptr(),
             self.out.data_ptr(), self.T, H, I, E, TOPK, 1, self.ws.buffer.data_ptr(),
             self.ctypes.c_size_t(self.ws.buffer.numel()), flags | self.base_flags,
             self.torch.cuda.current_stream().cuda_stream)
@@ -138,6 +150,18 @@ def time_calls(torch, fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall_ms
 
 
+def latency_percentiles(torch, fn, calls):
+    """p10 / p50 / p90 of single calls in microseconds, each between its own pair of events."""
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(calls)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    us = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+    return {"p10": us[len(us) // 10], "p50": us[len(us) // 2], "p90": us[(len(us) * 9) // 10], "calls": calls}
+
+
 def layer_bytes(T, n_active):
     """Algorithmic HBM bytes of one layer call: active expert weights once, x in, out, logits."""
     return n_active * 3 * H * I * 2 + 2 * T * H * 2 + T * E * 2
@@ -155,6 +179,7 @@ def measure(torch, T, w13, w2, steps, warmup, logits="normal"):
     torch.cuda.synchronize()
     na = run.n_active()
     ms, wall_ms = time_calls(torch, run, steps, warmup)
+    pct = latency_percentiles(torch, run, min(steps, 100))
     only = lambda keep: (_lib.FLAG_SKIP_ROUTER | _lib.FLAG_SKIP_ALIGN | _lib.FLAG_SKIP_GEMM1 |
                          _lib.FLAG_SKIP_GEMM2 | _lib.FLAG_SKIP_COMBINE) & ~keep
     stage = {}
@@ -162,7 +187,7 @@ def measure(torch, T, w13, w2, steps, warmup, logits="normal"):
                        ("router", _lib.FLAG_SKIP_ROUTER), ("align", _lib.FLAG_SKIP_ALIGN),
                        ("combine", _lib.FLAG_SKIP_COMBINE)):
         stage[name] = time_calls(torch, lambda f=only(flag): run(f), steps, max(2, warmup // 4))[0]
-    return {"T": T, "logits": logits, "ms": ms, "wall_ms": wall_ms, "n_active": na, "stage_ms": stage,
+    return {"T": T, "logits": logits, "ms": ms, "wall_ms": wall_ms, "n_active": na, "stage_ms": stage, "latency_us": pct,
             "tokens_per_s": T / ms * 1e3, "hbm_gbs": layer_bytes(T, na) / ms / 1e6,
             "tflops": layer_flops(T) / ms / 1e9}
 
@@ -254,6 +279,8 @@ def main():
         LayerRunner.base_flags = _lib.FLAG_W2_F16
     if args.wide_range:
         LayerRunner.base_flags |= _lib.FLAG_WIDE_RANGE
+    LayerRunner.extra_weight_sets = [tuple(t.to(w2.dtype) if i else t for i, t in enumerate(make_weights(torch, dev, seed=s)))
+                                     for s in range(1, args.weight_sets)]
 
     T = args.tokens
     head = measure(torch, T, w13, w2, args.steps, args.warmup)
@@ -299,8 +326,8 @@ def main():
         "config": {"workload": f"Mixtral-{args.shape} MoE layer T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
                                f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
                    "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate or args.w2_f16),
-                   "w2_dtype": "f16" if args.w2_f16 else "bf16"},
-        "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
+                   "w2_dtype": "f16" if args.w2_f16 else "bf16", "weight_sets": args.weight_sets},
+        "latency_us": head["latency_us"], "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(torch, T, w13, w2),
         "table": table,
