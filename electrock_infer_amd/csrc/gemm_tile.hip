@@ -444,8 +444,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                 const int c = tid + i * kThreads;  // 16-byte piece c of the tile: row c/16, columns (c%16)*8..+8
                 const int row = c >> 4;
                 if (row < valid)
-                    *reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + nt * 128 + (c & 15) * 8) =
-                        *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + (c & 15) * 16);
+                    // (non-temporal: the tile is not read again before the w2 GEMM; as ordinary stores the activations
+                    // displace weight and token lines, T=400-512: +3 % on this kernel)
+                    __builtin_nontemporal_store(
+                        *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + (c & 15) * 16),
+                        reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + nt * 128 + (c & 15) * 8));
             }
         }
     } else {
@@ -479,9 +482,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                 if (slot >= 0) {
                     const int64_t at = static_cast<int64_t>(slot) * p.H + (lane & 15) * 4;
                     if (p.y_f16)
-                        *reinterpret_cast<u32x2_t*>(ybase_h + at) = u32x2_t{pack_f16_sat(val[0], val[1]), pack_f16_sat(val[2], val[3])};
+                        __builtin_nontemporal_store(u32x2_t{pack_f16_sat(val[0], val[1]), pack_f16_sat(val[2], val[3])},
+                                                    reinterpret_cast<u32x2_t*>(ybase_h + at));
                     else
-                        *reinterpret_cast<f32x4_t*>(ybase + at) = val;
+                        __builtin_nontemporal_store(val, reinterpret_cast<f32x4_t*>(ybase + at));
                 }
             }
             __builtin_amdgcn_wave_barrier();

@@ -283,8 +283,11 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
                 const int c = tid + i * kThreads;
                 const int row = c / kPiecesRow, pc = c % kPiecesRow;
                 if (row < valid)
-                    *reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + col0 + nt * kColsC + pc * 8) =
-                        *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + pc * 16);
+                    // (non-temporal, as in the 256-row kernel: -2 to -3 % from 128 to 352 tokens; the same hint on the
+                    // partial sums of the w2 GEMM, which the combine reads at once, costs 1 %)
+                    __builtin_nontemporal_store(
+                        *reinterpret_cast<const u32x4_t*>(smem + row * kPitchC + pc * 16),
+                        reinterpret_cast<u32x4_t*>(dst + (m0 + row) * static_cast<int64_t>(p.I) + col0 + nt * kColsC + pc * 8));
             }
         }
     } else {
