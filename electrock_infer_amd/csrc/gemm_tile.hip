@@ -535,8 +535,10 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
         }
         attr_set[dev].store(true, std::memory_order_release);
     }
-    // one row tile per expert on average up to 7/8 full: weights are read once -> streaming copies
-    const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * 7;
+    // one row tile per expert on average up to 7/8 full: weights are read once -> streaming copies.  The w2 GEMM keeps
+    // them up to 1.25 row tiles per expert (T=1024-1280: -7 % on the kernel); the w13 GEMM does not: its streaming form
+    // also starts the tiles at different K offsets, which costs 8 % once most experts have two row tiles that share weights.
+    const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * (mode == 1 ? 7 : 10);
     const dim3 grid1(grid, 1), grid2(grid, static_cast<unsigned>(p.ksplit));
     auto go = [&](auto kernel, dim3 g, int kslice) {
         hipLaunchKernelGGL(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice);

@@ -435,7 +435,7 @@ def test_layer_mid_kernel_many_column_tiles(T, I, routing):
 
 
 @pytest.mark.parametrize("T", [8, 9, 16, 17, 63, 64, 191, 192, 193, 351, 352, 353, 447, 448, 449, 895, 896, 897,
-                               1023, 1024, 1025, 2047, 2048, 2049])
+                               1023, 1024, 1025, 1279, 1280, 1281, 2047, 2048, 2049])
 def test_layer_at_every_kernel_switch(T):
     """The batch sizes on both sides of every point where the layer changes kernels, K slices, sorted block,
     routing front or the format of the partial results."""
