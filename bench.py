@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Mixtral-8x7B MoE layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T] [--shape 8x7b|8x22b] [--accurate | --w2-f16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T] [--shape 8x7b|8x22b] [--mode MODE]
                     [--no-cpu] [--no-table]
 
 A "step" is one call of the layer (router, expert sort, w13 GEMM + SiLU*mul,
@@ -9,15 +9,25 @@ w2 GEMM, top-k combine) on one batch of T tokens resident in HBM.  The headline
 workload is the decode batch T=64 of the 8x7B shape (H=4096, I=14336, E=8,
 top-2 renormalised, bf16, N(0,1) router logits); `value` is T / (time per step).
 
+Modes (flag sets of em_moe_forward; every row of the output names its mode and carries the
+errors of that very mode against the fp32 oracle on sampled tokens):
+  default_f32out   flags = EM_FLAG_OUT_F32: the library's default arithmetic with a float32
+                   output -- the form the stated tolerance (max-abs 2e-2, mean relative 1e-3
+                   against an fp32 reference) is defined on.  The headline.
+  default          flags = 0: the same with the bf16 output the drop-in FusedMoE.forward returns
+                   (the output rounding alone is 1.4e-3 mean relative)
+  bf16_act         EM_FLAG_BF16_ACT: activations stored as bf16 between the GEMMs (the reference's type)
+  bf16_act_f16_partials  ... plus EM_FLAG_F16_PARTIALS: the fastest form for large batches
+  w2_f16_f32out    EM_FLAG_W2_F16 | EM_FLAG_OUT_F32: w2 converted to fp16 once by the caller
+
 One JSON line is printed.  Besides the contract fields it carries
   roofline      the dominant kernel (w13 GEMM + SiLU*mul), timed alone with HIP
                 events on the stream it is launched on, against 8 TB/s of HBM
   cpu_baseline  the reference-style torch CPU expert loop (oracle port) timed on
                 the host cores on the same workload
   latency_us    p10 / p50 / p90 of single layer calls, each between its own pair of events
-  table         layer latency / HBM GB/s / MFMA TFLOP/s for the other batch sizes
-                of the decode list, the headline batch in accurate mode and the
-                T=8192 prefill cases
+  table         layer latency / HBM GB/s / MFMA TFLOP/s / errors for the other batch sizes
+                (decode list, 512-2048 tokens, the T=8192 prefill routings) and the other modes
 """
 import argparse
 import json
@@ -44,17 +54,13 @@ def parse_args():
     ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
     ap.add_argument("--shape", choices=["8x7b", "8x22b"], default="8x7b",
                     help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
-    ap.add_argument("--accurate", action="store_true",
-                    help="run the layer with EM_FLAG_ACCURATE (SiLU*mul activations kept as fp16 instead of bf16 through the "
-                         "w2 GEMM)")
+    ap.add_argument("--mode", choices=sorted(MODES), default="default_f32out",
+                    help="flag set of the headline workload (see the module docstring)")
+    ap.add_argument("--no-errors", action="store_true",
+                    help="skip the error measurement against the fp32 oracle (it copies the weights to the host)")
     ap.add_argument("--weight-sets", type=int, default=1,
                     help="cycle the calls through N independently drawn sets of expert weights (N x 2.8 GB), so that no "
                          "call finds the weights of the one before in a cache")
-    ap.add_argument("--wide-range", action="store_true",
-                    help="EM_FLAG_WIDE_RANGE: float32 partial sums of the w2 GEMM at every batch size")
-    ap.add_argument("--w2-f16", action="store_true",
-                    help="hand w2 over as float16 (converted once from the bf16 weights): accurate mode's arithmetic "
-                         "without the conversion inside the w2 kernels")
     ap.add_argument("--operands", choices=["gaussian", "zeros"], default="gaussian",
                     help="values of x and the expert weights.  'zeros' is a diagnostic: the matrix pipes then draw "
                          "little power and the same kernels run at the full shader clock, which separates the "
@@ -69,6 +75,15 @@ def parse_args():
 
 
 OPERANDS = "gaussian"
+# mode name -> flags of em_moe_forward (numeric values of include/electrock_moe.h)
+F_OUT_F32, F_W2_F16, F_BF16_ACT, F_F16_PARTIALS = 1 << 0, 1 << 3, 1 << 5, 1 << 6
+MODES = {
+    "default_f32out": F_OUT_F32,
+    "default": 0,
+    "bf16_act": F_BF16_ACT,
+    "bf16_act_f16_partials": F_BF16_ACT | F_F16_PARTIALS,
+    "w2_f16_f32out": F_W2_F16 | F_OUT_F32,
+}
 
 
 def make_weights(torch, dev, seed=0):
@@ -102,18 +117,18 @@ def make_batch(torch, dev, T, seed=0, logits="normal"):
 class LayerRunner:
     """Calls em_moe_forward through the C ABI with pre-allocated buffers."""
 
-    base_flags = 0
     extra_weight_sets = []      # [(w13, w2), ...] cycled through together with the set given to the constructor
 
-    def __init__(self, torch, T, w13, w2, x, lg):
+    def __init__(self, torch, T, w13, w2, x, lg, mode_flags):
         import ctypes
         from electrock_infer_amd import _lib
         from electrock_infer_amd.layers.moe.fused_moe import MoeWorkspace
         self.torch, self._lib, self.ctypes = torch, _lib, ctypes
-        self.T, self.w13, self.w2, self.x, self.lg = T, w13, w2, x, lg
+        self.T, self.w13, self.x, self.lg, self.mode_flags = T, w13, x, lg, mode_flags
+        self.w2 = w2.to(torch.float16) if mode_flags & F_W2_F16 else w2
         self.more_sets, self.calls = LayerRunner.extra_weight_sets, 0
-        self.ws = MoeWorkspace(x.device, T, H, I, E, TOPK)
-        self.out = torch.empty_like(x)
+        self.ws = MoeWorkspace(x.device, T, H, I, E, TOPK, mode_flags)
+        self.out = torch.empty(T, H, device=x.device, dtype=torch.float32 if mode_flags & F_OUT_F32 else torch.bfloat16)
         self.lib = _lib.load()
 
     def __call__(self, flags=0):
@@ -123,10 +138,12 @@ class LayerRunner:
             self.calls += 1
             if k:
                 w13, w2 = self.more_sets[k - 1]
+                if self.mode_flags & F_W2_F16:
+                    w2 = w2.to(self.torch.float16)
         code = self.lib.em_moe_forward(
             self.x.data_ptr(), self.lg.data_ptr(), self._lib.DTYPE_BF16, w13.data_ptr(), w2.data_ptr(),
             self.out.data_ptr(), self.T, H, I, E, TOPK, 1, self.ws.buffer.data_ptr(),
-            self.ctypes.c_size_t(self.ws.buffer.numel()), flags | self.base_flags,
+            self.ctypes.c_size_t(self.ws.buffer.numel()), flags | self.mode_flags,
             self.torch.cuda.current_stream().cuda_stream)
         self._lib.check(code, "em_moe_forward")
 
@@ -171,35 +188,62 @@ def layer_flops(T):
     return T * TOPK * 6 * H * I
 
 
-def measure(torch, T, w13, w2, steps, warmup, logits="normal"):
+class HostWeights:
+    """fp32 copies of the expert weights on the host, for the oracle (error measurement and CPU baseline)."""
+
+    def __init__(self, w13, w2):
+        self.w13, self.w2 = w13.cpu().float(), w2.cpu().float()
+
+
+def layer_errors(torch, run, host, max_rows=64):
+    """max-abs and mean relative error of the runner's last output against the fp32 oracle on up to `max_rows`
+    tokens spread over the batch (the layer is token-wise).  Outside every timed region."""
+    from oracle import moe_oracle as O
+    T = run.T
+    rows = list(range(T)) if T <= max_rows else [int(i * (T - 1) / (max_rows - 1)) for i in range(max_rows)]
+    idx = torch.as_tensor(rows, device=run.x.device)
+    ref = O.moe_layer_fp32(run.x[idx].float().cpu(), run.lg[idx].float().cpu(), host.w13, host.w2)
+    d = (run.out[idx].double().cpu() - ref.double()).abs()
+    return {"max_abs": float(d.max()), "mean_rel": float(d.mean() / ref.double().abs().mean()), "rows": len(rows),
+            "against": "oracle.moe_layer_fp32"}
+
+
+def measure(torch, T, w13, w2, steps, warmup, logits="normal", mode="default_f32out", host=None, stages=True):
     from electrock_infer_amd import _lib
     x, lg = make_batch(torch, w13.device, T, logits=logits)
-    run = LayerRunner(torch, T, w13, w2, x, lg)
+    run = LayerRunner(torch, T, w13, w2, x, lg, MODES[mode])
     run()
     torch.cuda.synchronize()
     na = run.n_active()
+    errors = layer_errors(torch, run, host) if host is not None and not run.more_sets else None
     ms, wall_ms = time_calls(torch, run, steps, warmup)
     pct = latency_percentiles(torch, run, min(steps, 100))
     only = lambda keep: (_lib.FLAG_SKIP_ROUTER | _lib.FLAG_SKIP_ALIGN | _lib.FLAG_SKIP_GEMM1 |
                          _lib.FLAG_SKIP_GEMM2 | _lib.FLAG_SKIP_COMBINE) & ~keep
     stage = {}
-    for name, flag in (("gemm1", _lib.FLAG_SKIP_GEMM1), ("gemm2", _lib.FLAG_SKIP_GEMM2),
-                       ("router", _lib.FLAG_SKIP_ROUTER), ("align", _lib.FLAG_SKIP_ALIGN),
-                       ("combine", _lib.FLAG_SKIP_COMBINE)):
-        stage[name] = time_calls(torch, lambda f=only(flag): run(f), steps, max(2, warmup // 4))[0]
-    return {"T": T, "logits": logits, "ms": ms, "wall_ms": wall_ms, "n_active": na, "stage_ms": stage, "latency_us": pct,
-            "tokens_per_s": T / ms * 1e3, "hbm_gbs": layer_bytes(T, na) / ms / 1e6,
-            "tflops": layer_flops(T) / ms / 1e9}
+    if stages:
+        for name, flag in (("gemm1", _lib.FLAG_SKIP_GEMM1), ("gemm2", _lib.FLAG_SKIP_GEMM2),
+                           ("router", _lib.FLAG_SKIP_ROUTER), ("align", _lib.FLAG_SKIP_ALIGN),
+                           ("combine", _lib.FLAG_SKIP_COMBINE)):
+            stage[name] = time_calls(torch, lambda f=only(flag): run(f), steps, max(2, warmup // 4))[0]
+    r = {"T": T, "logits": logits, "mode": mode, "ms": ms, "wall_ms": wall_ms, "n_active": na, "stage_ms": stage,
+         "latency_us": pct, "tokens_per_s": T / ms * 1e3, "hbm_gbs": layer_bytes(T, na) / ms / 1e6,
+         "tflops": layer_flops(T) / ms / 1e9, "errors": errors}
+    r["hbm_frac"] = r["hbm_gbs"] / HBM_PEAK_GBS
+    r["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
+    if errors is not None:
+        r["meets_tolerance"] = bool(errors["max_abs"] <= 2e-2 and errors["mean_rel"] <= 1e-3)
+    return r
 
 
-def cpu_baseline(torch, T, w13, w2):
+def cpu_baseline(torch, T, w13, host):
     """Reference-style torch CPU expert loop (oracle port) on the same workload, host cores."""
     from oracle import moe_oracle as O
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
     torch.set_num_threads(cores)
     x, lg = make_batch(torch, w13.device, T)
     xc, lc = x.float().cpu(), lg.float().cpu()
-    w13c, w2c = w13.cpu().float(), w2.cpu().float()      # the CPU path holds fp32 weights
+    w13c, w2c = host.w13, host.w2                        # the CPU path holds fp32 weights
     O.moe_layer_fp32(xc, lc, w13c, w2c)                  # warm-up
     iters, t0 = 0, time.perf_counter()
     while iters < 3 or (time.perf_counter() - t0 < 10.0 and iters < 200):
@@ -213,13 +257,19 @@ def cpu_baseline(torch, T, w13, w2):
 
 def measured_traffic(T):
     """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
-    (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration), or None."""
+    (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration) and where that figure comes from; (None, None)
+    when no summary covers this batch size.  It is a property of the kernel, measured in profiler runs of their
+    own (counters cannot be read inside this process), not of this run."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(f"T{T}", {}).get("dominant_kernel_hbm_bytes")
+            entry = json.load(f).get(f"T{T}")
     except (OSError, ValueError):
-        return None
+        return None, None
+    if not entry:
+        return None, None
+    src = {k: entry.get(k) for k in ("dominant_kernel", "measured", "library_version", "summary")}
+    return entry.get("dominant_kernel_hbm_bytes"), src
 
 
 def calibrate_copy(torch, dev):
@@ -266,57 +316,51 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.accurate:
-        LayerRunner.base_flags = _lib.FLAG_ACCURATE
     if args.calibrate_copy:
         calibrate_copy(torch, dev)
     if args.vendor_gemm:
         print(json.dumps(vendor_gemm(torch, dev, args.tokens, min(args.steps, 30), min(args.warmup, 5))))
         return
     w13, w2 = make_weights(torch, dev)
-    if args.w2_f16:
-        w2 = w2.to(torch.float16)
-        LayerRunner.base_flags = _lib.FLAG_W2_F16
-    if args.wide_range:
-        LayerRunner.base_flags |= _lib.FLAG_WIDE_RANGE
-    LayerRunner.extra_weight_sets = [tuple(t.to(w2.dtype) if i else t for i, t in enumerate(make_weights(torch, dev, seed=s)))
-                                     for s in range(1, args.weight_sets)]
+    LayerRunner.extra_weight_sets = [make_weights(torch, dev, seed=s) for s in range(1, args.weight_sets)]
+    need_host = not (args.no_cpu and args.no_errors) and OPERANDS == "gaussian"
+    host = HostWeights(w13, w2) if need_host else None
+    err_host = None if args.no_errors else host
 
     T = args.tokens
-    head = measure(torch, T, w13, w2, args.steps, args.warmup)
+    head = measure(torch, T, w13, w2, args.steps, args.warmup, mode=args.mode, host=err_host)
     g1_ms = head["stage_ms"]["gemm1"]
+    traffic, traffic_src = measured_traffic(T)
     if T <= 1024:
         # decode: the w13 GEMM streams 2/3 of the weight bytes; HBM-bound
         g1_bytes = head["n_active"] * 2 * I * H * 2 + T * H * 2   # w13 of the active experts + x
         roofline = {"kernel": "w13 GEMM + SiLU*mul", "bound": "hbm", "achieved": g1_bytes / g1_ms / 1e6,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": measured_traffic(T),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": traffic, "traffic_source": traffic_src,
                     "per_launch": g1_bytes, "avg_launch_ms": g1_ms}
     else:
         # prefill: 4*H*I flops per routed slot in the w13 GEMM; MFMA-bound
         g1_flops = T * TOPK * 4 * H * I
         roofline = {"kernel": "w13 GEMM + SiLU*mul", "bound": "mfma", "achieved": g1_flops / g1_ms / 1e9,
-                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "traffic": measured_traffic(T),
+                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "traffic": traffic, "traffic_source": traffic_src,
                     "per_launch": g1_flops, "avg_launch_ms": g1_ms}
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
 
     table = []
     if not args.no_table:
-        for t in ((1, 8, 32, 64, 256) if args.shape == "8x7b" else (1, 64)):
-            if t != T:
-                table.append(measure(torch, t, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2)))
-        if not args.accurate and not args.w2_f16:  # the headline batch in accurate mode (fp16 activations)
-            from electrock_infer_amd import _lib
-            LayerRunner.base_flags = _lib.FLAG_ACCURATE
-            r = measure(torch, T, w13, w2, max(20, args.steps // 2), max(5, args.warmup // 2))
-            LayerRunner.base_flags = 0
-            r["accurate_mode"] = True
-            table.append(r)
+        half_steps, half_warm = max(20, args.steps // 2), max(5, args.warmup // 2)
+        big = 8192 if args.shape == "8x7b" else 4096
+        # the tolerance-meeting mode at every named batch size
+        for t in ((1, 8, 32, 64, 256, 512, 1024, 2048) if args.shape == "8x7b" else (1, 64)):
+            if t != T or args.mode != "default_f32out":
+                table.append(measure(torch, t, w13, w2, half_steps if t <= 256 else 20, half_warm, host=err_host))
         for lgk in (("normal", "zipf", "two_experts") if args.shape == "8x7b" else ("normal",)):
-            r = measure(torch, 8192 if args.shape == "8x7b" else 4096, w13, w2, 10, 3, logits=lgk)
-            r["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
-            table.append(r)
-    for r in [head] + table:
-        r["hbm_frac"] = r["hbm_gbs"] / HBM_PEAK_GBS
+            table.append(measure(torch, big, w13, w2, 10, 3, logits=lgk, host=err_host))
+        # the other modes at the headline batch and at the prefill batch
+        for mode in ("default", "bf16_act", "w2_f16_f32out"):
+            if mode != args.mode:
+                table.append(measure(torch, T, w13, w2, half_steps, half_warm, mode=mode, host=err_host, stages=False))
+        for mode in ("default", "bf16_act_f16_partials", "w2_f16_f32out"):
+            table.append(measure(torch, big, w13, w2, 10, 3, mode=mode, host=err_host))
 
     result = {
         "metric": f"Mixtral-{args.shape.upper().replace('X', 'x')} MoE layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s",
@@ -325,11 +369,12 @@ def main():
         "data": "synthetic" if args.operands == "gaussian" else "synthetic, all-zero x and weights (diagnostic)",
         "config": {"workload": f"Mixtral-{args.shape} MoE layer T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
                                f"x~N(0,1), weights~N(0,0.02), router logits~N(0,1), all experts resident",
-                   "tokens": T, "n_active_experts": head["n_active"], "accurate_mode": bool(args.accurate or args.w2_f16),
-                   "w2_dtype": "f16" if args.w2_f16 else "bf16", "weight_sets": args.weight_sets},
+                   "tokens": T, "n_active_experts": head["n_active"], "mode": args.mode, "flags": MODES[args.mode],
+                   "errors_vs_fp32_oracle": head["errors"], "meets_tolerance_2e-2_1e-3": head.get("meets_tolerance"),
+                   "w2_dtype": "f16" if MODES[args.mode] & F_W2_F16 else "bf16", "weight_sets": args.weight_sets},
         "latency_us": head["latency_us"], "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
         "roofline": roofline,
-        "cpu_baseline": None if args.no_cpu else cpu_baseline(torch, T, w13, w2),
+        "cpu_baseline": None if (args.no_cpu or host is None) else cpu_baseline(torch, T, w13, host),
         "table": table,
     }
     print(json.dumps(result))

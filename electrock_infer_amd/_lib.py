@@ -16,10 +16,10 @@ ITYPE_I32, ITYPE_I64 = 0, 1
 NORM_LAYER, NORM_OP = 0, 1   # rounding points of layers/layernorm.py resp. of the native add_rms_norm op
 
 FLAG_OUT_F32 = 1 << 0
-FLAG_ACCURATE = 1 << 1
 FLAG_GATE_F32_LOGITS = 1 << 2
 FLAG_W2_F16 = 1 << 3
-FLAG_WIDE_RANGE = 1 << 4
+FLAG_BF16_ACT = 1 << 5        # SiLU*mul activations stored as bf16 between the GEMMs (the reference's storage type)
+FLAG_F16_PARTIALS = 1 << 6    # bf16 output of large batches: w2 partial sums stored as fp16
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10
@@ -71,9 +71,9 @@ def load() -> ctypes.CDLL:
     lib.em_moe_sum.restype = i32
     lib.em_moe_sum.argtypes = [vp, vp, i64, i32, i64, i32, vp]
     lib.em_moe_workspace_bytes.restype = sz
-    lib.em_moe_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
+    lib.em_moe_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, u32]
     lib.em_moe_workspace_layout.restype = i32
-    lib.em_moe_workspace_layout.argtypes = [i64, i32, i32, i32, i32, ctypes.POINTER(MoeLayout)]
+    lib.em_moe_workspace_layout.argtypes = [i64, i32, i32, i32, i32, u32, ctypes.POINTER(MoeLayout)]
     lib.em_moe_forward.restype = i32
     lib.em_moe_forward.argtypes = [vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
     lib.em_moe_forward_gated.restype = i32
@@ -121,7 +121,7 @@ def require_device(*tensors) -> None:
             raise RuntimeError("tensor must be contiguous")
 
 
-def workspace_layout(T: int, H: int, I: int, E: int, top_k: int) -> MoeLayout:
+def workspace_layout(T: int, H: int, I: int, E: int, top_k: int, flags: int = 0) -> MoeLayout:
     L = MoeLayout()
-    check(load().em_moe_workspace_layout(T, H, I, E, top_k, ctypes.byref(L)), "em_moe_workspace_layout")
+    check(load().em_moe_workspace_layout(T, H, I, E, top_k, flags, ctypes.byref(L)), "em_moe_workspace_layout")
     return L

@@ -179,13 +179,13 @@ int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
     const dim3 grid(1), blk(kAlignThreads);
     if (itype == EM_ITYPE_I32) {
         if (E == 8)
-            hipLaunchKernelGGL((align_kernel<int32_t, 8>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
+            launch((align_kernel<int32_t, 8>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
                                numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
         else
-            hipLaunchKernelGGL((align_kernel<int32_t, 0>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
+            launch((align_kernel<int32_t, 0>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
                                numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else if (itype == EM_ITYPE_I64) {
-        hipLaunchKernelGGL((align_kernel<int64_t, 0>), grid, blk, 0, s, static_cast<const int64_t*>(ids),
+        launch((align_kernel<int64_t, 0>), grid, blk, 0, s, static_cast<const int64_t*>(ids),
                            numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
     } else {
         return EM_ERR_BAD_DTYPE;
@@ -200,7 +200,7 @@ int launch_route_align(const void* logits, int logits_dtype, int64_t T, int k, i
                        int32_t* post_pad, int32_t* seg_out, hipStream_t s) {
     const dim3 grid(1), blk(kAlignThreads);
     auto go = [&](auto kernel, auto* lp) {
-        hipLaunchKernelGGL(kernel, grid, blk, 0, s, lp, T, k, renorm, w, ids, block, sorted, sorted_len, expert_ids,
+        launch(kernel, grid, blk, 0, s, lp, T, k, renorm, w, ids, block, sorted, sorted_len, expert_ids,
                            eid_len, post_pad, seg_out);
     };
     switch (logits_dtype) {

@@ -6,7 +6,7 @@ using namespace em;
 
 namespace {
 
-constexpr int kVersion = 100;
+constexpr int kVersion = 200;
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 inline bool dtype_ok(int d) { return d == EM_DTYPE_F32 || d == EM_DTYPE_BF16 || d == EM_DTYPE_F16; }
@@ -58,6 +58,74 @@ inline int choose_ksplit(int64_t T, int H, int I) {
 bool shapes_ok(int64_t T, int H, int I, int E, int top_k) {
     return T >= 0 && H > 0 && I > 0 && E >= 1 && E <= kMaxExperts && top_k >= 1 && top_k <= kMaxTopK &&
            top_k <= E && H % 8 == 0 && I % 8 == 0 && T * top_k < (int64_t(1) << 30);
+}
+
+constexpr unsigned kKnownFlags = EM_FLAG_OUT_F32 | EM_FLAG_GATE_F32_LOGITS | EM_FLAG_W2_F16 | EM_FLAG_BF16_ACT |
+                                 EM_FLAG_F16_PARTIALS | EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN | EM_FLAG_SKIP_GEMM1 |
+                                 EM_FLAG_SKIP_GEMM2 | EM_FLAG_SKIP_COMBINE | EM_FLAG_FORCE_GENERIC;
+
+// What a layer call of these shapes and flags runs: which kernels, which storage types between them.  The
+// workspace layout and the stage sequencing both follow from it.
+struct Plan {
+    int block;
+    int ksplit;
+    int64_t sorted_len;
+    bool use_stream, use_tile;  // neither: the shape-generic kernels
+    bool w2_on_mid;             // streaming-size batch whose w2 GEMM runs on the 64-row tiled kernel
+    bool act_f16;               // SiLU*mul activations stored as fp16 (tuned kernels, default)
+    bool act_pair;              // ... as a bf16 pair (value, rounding residual): generic kernels, default
+    bool y_f16;                 // w2 partial sums stored as fp16 (opt-in, 256-row kernel, bf16 output)
+};
+
+Plan make_plan(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
+    Plan pl{};
+    pl.block = choose_block(T, H, I);
+    pl.ksplit = choose_ksplit(T, H, I);
+    pl.sorted_len = round_up(T * top_k + static_cast<int64_t>(E) * (pl.block - 1), pl.block);
+    MoeProblem q{};  // the fields the kernels' own shape checks read
+    q.T = T;
+    q.H = H;
+    q.I = I;
+    q.E = E;
+    q.top_k = top_k;
+    q.block = pl.block;
+    q.ksplit = pl.ksplit;
+    q.sorted_len = pl.sorted_len;
+    const bool tuned = !(flags & EM_FLAG_FORCE_GENERIC);
+    pl.use_stream = tuned && T <= kStreamMaxT && stream_supported(q);
+    pl.use_tile = tuned && T > kStreamMaxT && tile_supported(q);
+    pl.w2_on_mid = pl.use_stream && T > kStreamW2MaxT && pl.ksplit >= 2 && tile_mid_supported(q);
+    const bool bf16_act = (flags & EM_FLAG_BF16_ACT) != 0;
+    pl.act_f16 = !bf16_act && (pl.use_stream || pl.use_tile);
+    pl.act_pair = !bf16_act && !pl.act_f16;
+    pl.y_f16 = (flags & EM_FLAG_F16_PARTIALS) && !(flags & EM_FLAG_OUT_F32) && pl.use_tile && T > kTile128W2MaxT;
+    return pl;
+}
+
+int layout_from_plan(const Plan& pl, int64_t T, int H, int I, int E, int top_k, em_moe_layout* L) {
+    const int64_t slots = T * top_k;
+    int64_t off = 0;
+    auto take = [&off](int64_t bytes) {
+        const int64_t at = off;
+        off += round_up(bytes > 0 ? bytes : 1, 256);
+        return at;
+    };
+    L->block_size = pl.block;
+    L->topk_weights_off = take(slots * 4);
+    L->topk_ids_off = take(slots * 4);
+    L->sorted_ids_off = take(pl.sorted_len * 4);
+    L->sorted_len = pl.sorted_len;
+    L->expert_ids_len = pl.sorted_len / pl.block;
+    L->expert_ids_off = take(L->expert_ids_len * 4);
+    L->post_pad_off = take(4);
+    L->seg_begin_off = take((E + 1) * 4);
+    L->act_off = take(pl.sorted_len * static_cast<int64_t>(I) * 2);
+    // the rounding residuals exist only where the shape-generic kernels run in the default (two-term) form
+    L->act_lo_off = pl.act_pair ? take(pl.sorted_len * static_cast<int64_t>(I) * 2) : -1;
+    L->ksplit = pl.ksplit;
+    L->y_off = take(pl.ksplit * slots * static_cast<int64_t>(H) * 4);
+    L->total_bytes = off;
+    return 0;
 }
 
 }  // namespace
@@ -144,38 +212,16 @@ int em_add_rms_norm(const void* x_in, const void* residual_in, void* x_out, void
                            weight_dtype, semantics == EM_NORM_LAYER, as_stream(stream));
 }
 
-int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, em_moe_layout* L) {
+int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, unsigned flags, em_moe_layout* L) {
     if (!L) return EM_ERR_NULL_POINTER;
     if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
-    const int64_t block = choose_block(T, H, I);
-    const int64_t slots = T * top_k;
-    const int64_t sorted_len = round_up(slots + static_cast<int64_t>(E) * (block - 1), block);
-    int64_t off = 0;
-    auto take = [&off](int64_t bytes) {
-        const int64_t at = off;
-        off += round_up(bytes > 0 ? bytes : 1, 256);
-        return at;
-    };
-    L->block_size = block;
-    L->topk_weights_off = take(slots * 4);
-    L->topk_ids_off = take(slots * 4);
-    L->sorted_ids_off = take(sorted_len * 4);
-    L->sorted_len = sorted_len;
-    L->expert_ids_len = sorted_len / block;
-    L->expert_ids_off = take(L->expert_ids_len * 4);
-    L->post_pad_off = take(4);
-    L->seg_begin_off = take((E + 1) * 4);
-    L->act_off = take(sorted_len * static_cast<int64_t>(I) * 2);
-    L->act_lo_off = take(sorted_len * static_cast<int64_t>(I) * 2);
-    L->ksplit = choose_ksplit(T, H, I);
-    L->y_off = take(L->ksplit * slots * static_cast<int64_t>(H) * 4);
-    L->total_bytes = off;
-    return 0;
+    if (flags & ~kKnownFlags) return EM_ERR_UNSUPPORTED;
+    return layout_from_plan(make_plan(T, H, I, E, top_k, flags), T, H, I, E, top_k, L);
 }
 
-size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k) {
+size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
     em_moe_layout L;
-    if (em_moe_workspace_layout(T, H, I, E, top_k, &L) != 0) return 0;
+    if (em_moe_workspace_layout(T, H, I, E, top_k, flags, &L) != 0) return 0;
     return static_cast<size_t>(L.total_bytes);
 }
 
@@ -210,8 +256,12 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     if (!aligned(x, 16) || !aligned(w13, 16) || !aligned(w2, 16) || !aligned(out, 16) ||
         !aligned(workspace, 256))
         return EM_ERR_ALIGNMENT;
+    if (flags & ~kKnownFlags) return EM_ERR_UNSUPPORTED;
+    const Plan pl = make_plan(T, H, I, E, top_k, flags);
+    // fp16 w2: only the tuned kernels have an fp16 w2 GEMM, and it multiplies fp16 activations
+    if ((flags & EM_FLAG_W2_F16) && (!pl.act_f16)) return EM_ERR_UNSUPPORTED;
     em_moe_layout L;
-    int rc = em_moe_workspace_layout(T, H, I, E, top_k, &L);
+    int rc = layout_from_plan(pl, T, H, I, E, top_k, &L);
     if (rc != 0) return rc;
     if (workspace_bytes < static_cast<size_t>(L.total_bytes)) return EM_ERR_WORKSPACE;
 
@@ -222,11 +272,20 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.w13 = static_cast<const uint16_t*>(w13);
     p.w2 = static_cast<const uint16_t*>(w2);
     p.act = reinterpret_cast<uint16_t*>(ws + L.act_off);
-    const bool accurate = (flags & (EM_FLAG_ACCURATE | EM_FLAG_W2_F16)) != 0;
-    p.act_lo = accurate ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
-    p.act_f16 = 0;
+    // The rounding of the SiLU*mul activations stays out of the result unless EM_FLAG_BF16_ACT asks for the
+    // reference's bf16 storage.  With the tuned kernels the activations are stored as fp16 (three more mantissa bits
+    // than bf16; clamped to the fp16 range) and the w2 kernel turns its bf16 weight fragments into fp16 on their way
+    // to the MFMA: no extra traffic and no second pass.  The shape-generic kernels store a bf16 pair (value, residual)
+    // and multiply the residual in a second accumulating pass.
+    p.act_lo = pl.act_pair ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
+    p.act_f16 = pl.act_f16 ? 1 : 0;
     p.w2_f16 = (flags & EM_FLAG_W2_F16) ? 1 : 0;
-    p.y_f16 = 0;
+    // The partial results of the w2 GEMM (one per routed slot and K slice, before the routing weight) are float32.
+    // EM_FLAG_F16_PARTIALS stores those of the 256-row kernel as fp16 where the output is bf16 (their rounding, 2^-12,
+    // is far below the output's, 2^-9): half the bytes written by the kernel's epilogues, which all fall into the same
+    // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer) -- but fp16 saturates
+    // at 65504 where the reference's bf16 pipeline does not, so a caller has to ask for it.
+    p.y_f16 = pl.y_f16 ? 1 : 0;
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
@@ -248,9 +307,6 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.sorted_len = L.sorted_len;
     p.ksplit = static_cast<int>(L.ksplit);
 
-    // fp16 w2: only the tuned kernels have an fp16 w2 GEMM (checked before anything is launched)
-    if (p.w2_f16 && ((flags & EM_FLAG_FORCE_GENERIC) || !(T <= kStreamMaxT ? stream_supported(p) : tile_supported(p))))
-        return EM_ERR_UNSUPPORTED;
     const bool fused_front = !(flags & (EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN)) && norm == nullptr &&
                              gate_w == nullptr && route_align_supported(T, E, top_k);
     if (fused_front) {
@@ -275,23 +331,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
                           L.expert_ids_len, post_pad, seg_begin, s);
         if (rc != 0) return rc;
     }
-    const bool use_stream = !(flags & EM_FLAG_FORCE_GENERIC) && T <= kStreamMaxT && stream_supported(p);
-    const bool use_tile = !(flags & EM_FLAG_FORCE_GENERIC) && T > kStreamMaxT && tile_supported(p);
-    // Accurate mode keeps the rounding of the SiLU*mul activations out of the result.  With the tuned kernels the
-    // activations are stored as fp16 (three more mantissa bits than bf16; clamped to the fp16 range) and the w2
-    // kernel turns its bf16 weight fragments into fp16 on their way to the MFMA: no extra traffic and no second
-    // pass.  The shape-generic kernels store a bf16 pair (value, residual) and multiply the residual in a second
-    // accumulating pass.
-    const bool w2_on_mid = use_stream && T > kStreamW2MaxT && p.ksplit >= 2 && tile_mid_supported(p);
-    if (accurate && (use_stream || use_tile)) {
-        p.act_f16 = 1;
-        p.act_lo = nullptr;
-    }
-    // Where the output is bf16, the partial results of the 256-row w2 kernel are fp16 (their rounding, 2^-12, is far
-    // below the output's, 2^-9): half the bytes written by the kernel's epilogues, which all fall into the same
-    // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer).
-    // fp16 saturates at 65504: EM_FLAG_WIDE_RANGE keeps the partial results float32 for callers whose values may pass it.
-    if (use_tile && T > kTile128W2MaxT && !(flags & (EM_FLAG_OUT_F32 | EM_FLAG_WIDE_RANGE))) p.y_f16 = 1;
+    const bool use_stream = pl.use_stream, use_tile = pl.use_tile;
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
         if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
@@ -303,18 +343,18 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (rc != 0) return rc;
     }
     if (!(flags & EM_FLAG_SKIP_GEMM2)) {
-        if (w2_on_mid) {
+        if (pl.w2_on_mid) {
             rc = launch_gemm_tile_mid(p, seg_begin, 2, 64, s);
         } else if (use_stream) {
             rc = launch_gemm_stream(p, seg_begin, 2, s);
         } else {
             rc = use_tile ? tile_gemm(p, 2) : launch_gemm_generic(p, 2, s);
-            if (rc == 0 && accurate && !p.act_f16) {  // second pass: y += act_lo . w2
+            if (rc == 0 && pl.act_pair) {  // second pass: y += act_lo . w2
                 MoeProblem lo = p;
                 lo.act = p.act_lo;
                 lo.act_lo = nullptr;
                 lo.y_accumulate = 1;
-                rc = launch_gemm_generic(lo, 2, s);  // (the tuned kernels never get here: they take fp16 activations)
+                rc = launch_gemm_generic(lo, 2, s);
             }
         }
         if (rc != 0) return rc;

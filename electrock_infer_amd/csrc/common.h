@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <tuple>
+#include <utility>
 #include "../../include/electrock_moe.h"
 
 namespace em {
@@ -100,7 +102,32 @@ struct F16Elem {
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
-inline int launch_status() { return static_cast<int>(hipGetLastError()); }
+// Kernel launches report through the return value of hipLaunchKernel, not through the runtime's sticky
+// "last error": that one may hold an error of unrelated earlier work of the caller, and reading it clears it.
+// launch() notes a failed launch for the calling thread, launch_status() returns the first one noted since it
+// was last asked (0 = every launch was queued).
+inline int& launch_rc() {
+    static thread_local int rc = 0;
+    return rc;
+}
+template <typename... KArgs, size_t... Is>
+inline hipError_t launch_tuple(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s,
+                               std::tuple<KArgs...>& vals, std::index_sequence<Is...>) {
+    void* ptrs[] = {static_cast<void*>(&std::get<Is>(vals))...};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds, s);
+}
+template <typename... KArgs, typename... Args>
+inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s, Args&&... args) {
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "argument count does not match the kernel's");
+    std::tuple<KArgs...> vals(static_cast<KArgs>(std::forward<Args>(args))...);
+    const hipError_t e = launch_tuple(kernel, grid, block, lds, s, vals, std::index_sequence_for<KArgs...>{});
+    if (e != hipSuccess && launch_rc() == 0) launch_rc() = static_cast<int>(e);
+}
+inline int launch_status() {
+    const int rc = launch_rc();
+    launch_rc() = 0;
+    return rc;
+}
 
 // ---- stage launchers (defined in the .hip files, called from capi.hip) ------
 int launch_router(const void* logits, int logits_dtype, int64_t T, int E, int k, int renorm,

@@ -107,10 +107,10 @@ int run_silu(void* out, const void* in, int64_t rows, int64_t d, hipStream_t s) 
     const dim3 grid(static_cast<unsigned>(rows),
                     static_cast<unsigned>(ceil_div(work, kEwThreads) < 64 ? ceil_div(work, kEwThreads) : 64));
     if (vec)
-        hipLaunchKernelGGL((silu_and_mul_kernel<Elem, true>), grid, dim3(kEwThreads), 0, s,
+        launch((silu_and_mul_kernel<Elem, true>), grid, dim3(kEwThreads), 0, s,
                            static_cast<S*>(out), static_cast<const S*>(in), d);
     else
-        hipLaunchKernelGGL((silu_and_mul_kernel<Elem, false>), grid, dim3(kEwThreads), 0, s,
+        launch((silu_and_mul_kernel<Elem, false>), grid, dim3(kEwThreads), 0, s,
                            static_cast<S*>(out), static_cast<const S*>(in), d);
     return launch_status();
 }
@@ -124,10 +124,10 @@ int run_sum(const void* in, void* out, int64_t T, int topk, int64_t H, hipStream
     const dim3 grid(static_cast<unsigned>(T),
                     static_cast<unsigned>(ceil_div(work, kEwThreads) < 64 ? ceil_div(work, kEwThreads) : 64));
     if (vec)
-        hipLaunchKernelGGL((moe_sum_kernel<Elem, true>), grid, dim3(kEwThreads), 0, s,
+        launch((moe_sum_kernel<Elem, true>), grid, dim3(kEwThreads), 0, s,
                            static_cast<const S*>(in), static_cast<S*>(out), topk, H);
     else
-        hipLaunchKernelGGL((moe_sum_kernel<Elem, false>), grid, dim3(kEwThreads), 0, s,
+        launch((moe_sum_kernel<Elem, false>), grid, dim3(kEwThreads), 0, s,
                            static_cast<const S*>(in), static_cast<S*>(out), topk, H);
     return launch_status();
 }

@@ -77,9 +77,10 @@ constexpr int64_t kFusedNormMaxT = 16;  // up to here norm + gate + router share
 constexpr int kResidentSteps = 8;    // K steps of 32 a wave keeps in registers: 16 waves x 8 x 32 = 4096
 template <int E_, typename WElem, bool ADD, bool LAYER, bool RESIDENT>
 __global__ __launch_bounds__(kNormGateThreads) void norm_gate_router_kernel(
-    const uint16_t* __restrict__ x_in, const uint16_t* __restrict__ res_in,
-    const typename WElem::storage* __restrict__ norm_w, float eps, uint16_t* __restrict__ h_out,
-    uint16_t* __restrict__ res_out, const uint16_t* __restrict__ gate_w, int64_t T, int H, int k, int renorm,
+    // h_out may be x_in (plain norm, or norm of the sum with the residual written elsewhere): no __restrict__ on the rows
+    const uint16_t* x_in, const uint16_t* res_in,
+    const typename WElem::storage* __restrict__ norm_w, float eps, uint16_t* h_out,
+    uint16_t* res_out, const uint16_t* __restrict__ gate_w, int64_t T, int H, int k, int renorm,
     int round_bf16, void* __restrict__ logits_out, float* __restrict__ out_w, int32_t* __restrict__ out_ids) {
     static_assert(E_ == 8 || E_ == 16, "experts sit in the 16 rows of one MFMA");
     __shared__ __attribute__((aligned(16))) float partial[kNormGateWaves][kGateTokens][E_];
@@ -236,13 +237,13 @@ void launch_norm_gate(bool add, bool layer, unsigned grid, hipStream_t s, const 
     const WS* nwp = static_cast<const WS*>(nw);
     const dim3 gd(grid), bd(kNormGateThreads);
     if (add && layer)
-        hipLaunchKernelGGL((norm_gate_router_kernel<E_, WElem, true, true, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
+        launch((norm_gate_router_kernel<E_, WElem, true, true, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
     else if (add)
-        hipLaunchKernelGGL((norm_gate_router_kernel<E_, WElem, true, false, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
+        launch((norm_gate_router_kernel<E_, WElem, true, false, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
     else if (layer)
-        hipLaunchKernelGGL((norm_gate_router_kernel<E_, WElem, false, true, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
+        launch((norm_gate_router_kernel<E_, WElem, false, true, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
     else
-        hipLaunchKernelGGL((norm_gate_router_kernel<E_, WElem, false, false, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
+        launch((norm_gate_router_kernel<E_, WElem, false, false, RESIDENT>), gd, bd, 0, s, x, r, nwp, eps, h, ro, g, T, H, k, renorm, round_bf16, lo, w, ids);
 }
 
 }  // namespace
@@ -259,10 +260,10 @@ int launch_gate_router(const void* x, const void* gate_w, int64_t T, int H, int 
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const uint16_t* gp = static_cast<const uint16_t*>(gate_w);
     if (E == 8)
-        hipLaunchKernelGGL(gate_router_kernel<8>, dim3(grid), dim3(kGateThreads), 0, s, xp, gp, T, H, k, renorm,
+        launch(gate_router_kernel<8>, dim3(grid), dim3(kGateThreads), 0, s, xp, gp, T, H, k, renorm,
                            round_bf16, logits_out, w, ids);
     else
-        hipLaunchKernelGGL(gate_router_kernel<16>, dim3(grid), dim3(kGateThreads), 0, s, xp, gp, T, H, k, renorm,
+        launch(gate_router_kernel<16>, dim3(grid), dim3(kGateThreads), 0, s, xp, gp, T, H, k, renorm,
                            round_bf16, logits_out, w, ids);
     return launch_status();
 }

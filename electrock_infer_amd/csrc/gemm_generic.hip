@@ -261,9 +261,9 @@ int launch_gemm_generic(const MoeProblem& p, int mode, hipStream_t s) {
                                          static_cast<unsigned>(p.ksplit));
 #define EM_LAUNCH_GENERIC(MODE)                                                             \
     do {                                                                                    \
-        if (tile_rows == 16) hipLaunchKernelGGL((gemm_generic_kernel<MODE, 1>), grid, blk, 0, s, p);      \
-        else if (tile_rows == 32) hipLaunchKernelGGL((gemm_generic_kernel<MODE, 2>), grid, blk, 0, s, p); \
-        else hipLaunchKernelGGL((gemm_generic_kernel<MODE, 4>), grid, blk, 0, s, p);                      \
+        if (tile_rows == 16) launch((gemm_generic_kernel<MODE, 1>), grid, blk, 0, s, p);      \
+        else if (tile_rows == 32) launch((gemm_generic_kernel<MODE, 2>), grid, blk, 0, s, p); \
+        else launch((gemm_generic_kernel<MODE, 4>), grid, blk, 0, s, p);                      \
     } while (0)
     if (mode == 1) EM_LAUNCH_GENERIC(1);
     else EM_LAUNCH_GENERIC(2);
@@ -280,7 +280,7 @@ int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
         const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 2048));
         const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
         auto go = [&](auto kernel) {
-            hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.topk_w,
+            launch(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.topk_w,
                                static_cast<uint16_t*>(out), p.T, p.H, p.top_k, p.ksplit);
         };
         if (stream) go(combine_f16_kernel<true>); else go(combine_f16_kernel<false>);
@@ -289,7 +289,7 @@ int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
     const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 1024));
     const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
     auto go = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k, p.ksplit);
+        launch(kernel, grid, dim3(256), 0, s, p.y, p.topk_w, out, p.T, p.H, p.top_k, p.ksplit);
     };
     if (out_f32) { if (stream) go(combine_kernel<true, true>); else go(combine_kernel<true, false>); }
     else { if (stream) go(combine_kernel<false, true>); else go(combine_kernel<false, false>); }

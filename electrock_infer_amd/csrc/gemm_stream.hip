@@ -231,15 +231,15 @@ int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, 
     const dim3 blk(kWaves * 64);
     if (mode == 1) {
         const int tiles = p.I / 32;
-        hipLaunchKernelGGL((gemm_stream_kernel<1, false>), dim3(static_cast<unsigned>(p.E * tiles), 1), blk, 0, s, p,
+        launch((gemm_stream_kernel<1, false>), dim3(static_cast<unsigned>(p.E * tiles), 1), blk, 0, s, p,
                            seg_begin, tiles, p.H);
     } else {
         const int tiles = p.H / kRows;
         const dim3 grid(static_cast<unsigned>(p.E * tiles), static_cast<unsigned>(p.ksplit));
         if (p.act_f16)
-            hipLaunchKernelGGL((gemm_stream_kernel<2, true>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
+            launch((gemm_stream_kernel<2, true>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
         else
-            hipLaunchKernelGGL((gemm_stream_kernel<2, false>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
+            launch((gemm_stream_kernel<2, false>), grid, blk, 0, s, p, seg_begin, tiles, p.I / p.ksplit);
     }
     return launch_status();
 }

@@ -541,7 +541,7 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * (mode == 1 ? 7 : 10);
     const dim3 grid1(grid, 1), grid2(grid, static_cast<unsigned>(p.ksplit));
     auto go = [&](auto kernel, dim3 g, int kslice) {
-        hipLaunchKernelGGL(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice);
+        launch(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice);
     };
     if (mode == 1) {
         if (stream_b) go(gemm_tile_kernel<1, true, 0>, grid1, p.H);

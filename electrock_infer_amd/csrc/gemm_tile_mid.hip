@@ -366,7 +366,7 @@ int launch_mid(const MoeProblem& p, const int32_t* seg_begin, hipStream_t s) {
         if (e != hipSuccess) return static_cast<int>(e);
         attr_set[dev].store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((gemm_tile_mid_kernel<MODE, MI, F16>), dim3(grid, static_cast<unsigned>(slices)), dim3(kThreads),
+    launch((gemm_tile_mid_kernel<MODE, MI, F16>), dim3(grid, static_cast<unsigned>(slices)), dim3(kThreads),
                        kLdsBytes, s, p, seg_begin, wide_blocks, ntn_wide, col0n, ntn_narrow,
                        (MODE == 1) ? p.H : p.I / p.ksplit);
     return launch_status();

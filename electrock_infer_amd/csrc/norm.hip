@@ -25,9 +25,10 @@ template <typename Elem> struct NormVec { static constexpr int n = 16 / sizeof(t
 
 template <typename Elem, typename WElem, bool ADD, bool LAYER>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(
-    const typename Elem::storage* __restrict__ x_in, const typename Elem::storage* __restrict__ res_in,
-    const typename WElem::storage* __restrict__ weight, typename Elem::storage* __restrict__ x_out,
-    typename Elem::storage* __restrict__ res_out, int H, float eps) {
+    // x_out may be x_in and res_out may be res_in (the native op works in place): no __restrict__ on those four
+    const typename Elem::storage* x_in, const typename Elem::storage* res_in,
+    const typename WElem::storage* __restrict__ weight, typename Elem::storage* x_out,
+    typename Elem::storage* res_out, int H, float eps) {
     typedef typename Elem::storage S;
     typedef typename WElem::storage WS;
     constexpr int V = NormVec<Elem>::n;
@@ -120,13 +121,13 @@ int launch_typed(const void* x_in, const void* res_in, const void* weight, void*
     S* xo = static_cast<S*>(x_out);
     S* ro = static_cast<S*>(res_out);
     if (add && layer)
-        hipLaunchKernelGGL((rms_norm_kernel<Elem, WElem, true, true>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
+        launch((rms_norm_kernel<Elem, WElem, true, true>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
     else if (add)
-        hipLaunchKernelGGL((rms_norm_kernel<Elem, WElem, true, false>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
+        launch((rms_norm_kernel<Elem, WElem, true, false>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
     else if (layer)
-        hipLaunchKernelGGL((rms_norm_kernel<Elem, WElem, false, true>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
+        launch((rms_norm_kernel<Elem, WElem, false, true>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
     else
-        hipLaunchKernelGGL((rms_norm_kernel<Elem, WElem, false, false>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
+        launch((rms_norm_kernel<Elem, WElem, false, false>), grid, block, 0, s, xi, ri, w, xo, ro, H, eps);
     return launch_status();
 }
 

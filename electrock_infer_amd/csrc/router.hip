@@ -38,7 +38,7 @@ void launch_typed(const void* logits, int64_t T, int E, int k, int renorm, float
     const dim3 block(kRouterWaves * kWave);
     auto go = [&](auto kernel, int g) {
         const dim3 grid(static_cast<unsigned>(ceil_div(T, static_cast<int64_t>(kRouterWaves) * (kWave / g))));
-        hipLaunchKernelGGL(kernel, grid, block, 0, s, lp, T, E, k, renorm, w, ids);
+        launch(kernel, grid, block, 0, s, lp, T, E, k, renorm, w, ids);
     };
     if (E <= 8) go(router_kernel<Elem, 8>, 8);
     else if (E <= 16) go(router_kernel<Elem, 16>, 16);

@@ -6,7 +6,7 @@ meaning and return values; behind them sits one call into the C ABI
 (``em_topk_softmax`` / ``em_moe_forward``) instead of torch ops + Triton.
 """
 import ctypes
-from typing import Dict, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -40,19 +40,25 @@ def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: i
 
 
 class MoeWorkspace:
-    """Device scratch for ``em_moe_forward``, cached per (device, shape).
+    """Device scratch of one ``em_moe_forward`` call shape: a 256-byte aligned buffer plus the layout of the
+    call in it.
 
     The reference allocates its three intermediate caches and the sort buffers
     on every call (fused_moe.py:223-239, moe_align_block_size.py:32-48); here one
-    256-byte aligned buffer is kept and reused, and views of the routing results
-    the kernels leave in it can be read back for inspection.
+    buffer is kept and reused, and views of the routing results
+    the kernels leave in it can be read back for inspection.  ``buffer`` may be any
+    uint8 device tensor of at least ``layout.total_bytes`` (several shapes can share one).
     """
 
-    def __init__(self, device, T: int, H: int, I: int, E: int, top_k: int):
+    def __init__(self, device, T: int, H: int, I: int, E: int, top_k: int, flags: int = 0,
+                 buffer: Optional[torch.Tensor] = None):
         self.shape = (T, H, I, E, top_k)
-        self.layout = _lib.workspace_layout(T, H, I, E, top_k)
-        self.buffer = torch.empty(self.layout.total_bytes, dtype=torch.uint8, device=device)
-        assert self.buffer.data_ptr() % 256 == 0
+        self.layout = _lib.workspace_layout(T, H, I, E, top_k, flags & _LAYOUT_FLAGS)
+        if buffer is None:
+            buffer = torch.empty(self.layout.total_bytes, dtype=torch.uint8, device=device)
+        if buffer.numel() < self.layout.total_bytes or buffer.data_ptr() % 256 != 0:
+            raise RuntimeError("workspace buffer too small or not 256-byte aligned")
+        self.buffer = buffer
 
     def _view(self, off: int, count: int, dtype: torch.dtype) -> torch.Tensor:
         nbytes = count * torch.empty((), dtype=dtype).element_size()
@@ -80,26 +86,59 @@ class MoeWorkspace:
         return self._view(self.layout.post_pad_off, 1, torch.int32)
 
 
-_workspaces: Dict[tuple, MoeWorkspace] = {}
+# the flags the workspace size depends on
+_LAYOUT_FLAGS = _lib.FLAG_BF16_ACT | _lib.FLAG_FORCE_GENERIC
+
+# One grow-only buffer per device.  A buffer that has been handed out is never freed behind the caller's back:
+# a HIP graph captured through the layer calls holds its address, so when a larger batch makes the buffer grow,
+# the old one is kept (``_retired``) until ``release_workspaces``.  Growth is geometric, so the retired buffers
+# together stay below twice the live one; an engine that knows its largest batch calls ``reserve_workspace`` once.
+_buffers: Dict[int, torch.Tensor] = {}
+_retired: Dict[int, List[torch.Tensor]] = {}
 
 
-def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int) -> MoeWorkspace:
-    """The cached workspace of a device.  Calls on one device share it: they have to be ordered on one stream (as the
-    layers of a model are); a caller that runs layer calls on several streams at once passes each its own
-    ``MoeWorkspace`` through the ``workspace`` argument of the entry points."""
-    key = (torch.device(device).index, T, H, I, E, top_k)
-    ws = _workspaces.get(key)
-    if ws is None:
-        # keep one workspace per device: drop those of other batch sizes
-        for k in [k for k in _workspaces if k[0] == key[0]]:
-            del _workspaces[k]
-        ws = _workspaces[key] = MoeWorkspace(device, T, H, I, E, top_k)
-    return ws
+def _device_index(device) -> int:
+    d = torch.device(device)
+    return d.index if d.index is not None else torch.cuda.current_device()
+
+
+def _ensure_buffer(device, nbytes: int) -> torch.Tensor:
+    idx = _device_index(device)
+    buf = _buffers.get(idx)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _retired.setdefault(idx, []).append(buf)
+            nbytes = max(nbytes, buf.numel() * 3 // 2)
+        buf = _buffers[idx] = torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", idx))
+        assert buf.data_ptr() % 256 == 0
+    return buf
+
+
+def reserve_workspace(device, T: int, H: int, I: int, E: int, top_k: int, flags: int = 0) -> None:
+    """Size the device's shared workspace for calls of up to this shape (an engine: its largest batch), so that
+    no later call allocates."""
+    _ensure_buffer(device, _lib.workspace_layout(T, H, I, E, top_k, flags & _LAYOUT_FLAGS).total_bytes)
+
+
+def release_workspaces(device=None) -> None:
+    """Drop the shared workspaces (of one device, or of all): only when no captured graph and no pending call
+    uses them any more."""
+    for idx in ([_device_index(device)] if device is not None else list(_buffers)):
+        _buffers.pop(idx, None)
+        _retired.pop(idx, None)
+
+
+def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int, flags: int = 0) -> MoeWorkspace:
+    """The layout of a call of this shape in the device's shared workspace.  Calls on one device share that buffer:
+    they have to be ordered on one stream (as the layers of a model are); a caller that runs layer calls on several
+    streams at once passes each its own ``MoeWorkspace`` through the ``workspace`` argument of the entry points."""
+    need = _lib.workspace_layout(T, H, I, E, top_k, flags & _LAYOUT_FLAGS).total_bytes
+    return MoeWorkspace(device, T, H, I, E, top_k, flags, buffer=_ensure_buffer(device, need))
 
 
 def _w2_flag(w2: torch.Tensor) -> int:
     """w2 may be kept as float16 (converted once from the bfloat16 checkpoint, exactly for every weight of magnitude
-    2^-14 .. 65504): the layer then runs in accurate mode with no conversion in the w2 GEMM."""
+    2^-14 .. 65504): the w2 GEMM then needs no conversion of its weight fragments."""
     if w2.dtype == torch.float16:
         return _lib.FLAG_W2_F16
     if w2.dtype != torch.bfloat16:
@@ -110,7 +149,7 @@ def _w2_flag(w2: torch.Tensor) -> int:
 def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
                   gating_output: torch.Tensor, topk: int, renormalize: bool = True,
                   inplace: bool = False, activation: str = "silu",
-                  out_dtype: Optional[torch.dtype] = None, accurate: bool = False, flags: int = 0,
+                  out_dtype: Optional[torch.dtype] = None, bf16_act: bool = False, flags: int = 0,
                   workspace: Optional[MoeWorkspace] = None) -> torch.Tensor:
     """The MoE layer body (fused_moe.py:170-293): route, sort, w13 GEMM with
     SiLU*mul, w2 GEMM, weighted top-k combine.
@@ -119,9 +158,10 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     gating_output [T, E].  With ``inplace`` the result overwrites
     ``hidden_states`` and that tensor is returned, as in the reference.
     ``out_dtype=torch.float32`` returns the un-rounded fp32 result instead
-    (not available together with ``inplace``).  ``accurate=True`` keeps the
-    SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM; a float16
-    ``w2`` does the same without the conversion of the weights inside the kernel.
+    (not available together with ``inplace``).  Between the two GEMMs the
+    SiLU*mul activations are kept as fp16; ``bf16_act=True`` rounds them to
+    bf16 as the reference's ``cache2`` does (its range, its rounding error).  A float16
+    ``w2`` saves the conversion of the weight fragments inside the w2 kernel.
     """
     if activation != "silu":
         raise NotImplementedError(f"Activation {activation} not supported.")
@@ -137,8 +177,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, w1 and w2 must be bfloat16")
     flags |= _w2_flag(w2)
     want_f32 = out_dtype == torch.float32
-    if accurate:
-        flags |= _lib.FLAG_ACCURATE
+    if bf16_act:
+        flags |= _lib.FLAG_BF16_ACT
     if want_f32 and inplace:
         raise RuntimeError("a float32 result cannot be written in place over bfloat16 hidden_states")
     if want_f32:
@@ -148,7 +188,7 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         output = hidden_states if inplace else torch.empty_like(hidden_states)
     if T == 0:
         return output
-    ws = workspace or get_workspace(hidden_states.device, T, H, I, E, topk)
+    ws = workspace or get_workspace(hidden_states.device, T, H, I, E, topk, flags)
     code = _lib.load().em_moe_forward(
         hidden_states.data_ptr(), gating_output.data_ptr(), _lib.dtype_code(gating_output.dtype),
         w1.data_ptr(), w2.data_ptr(), output.data_ptr(), T, H, I, E, topk, 1 if renormalize else 0,
@@ -188,7 +228,7 @@ def gate_topk(hidden_states: torch.Tensor, gate_weight: torch.Tensor, topk: int,
 
 def fused_experts_gated(hidden_states: torch.Tensor, gate_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
                         topk: int, renormalize: bool = True, inplace: bool = False,
-                        out_dtype: Optional[torch.dtype] = None, accurate: bool = False, bf16_logits: bool = True,
+                        out_dtype: Optional[torch.dtype] = None, bf16_act: bool = False, bf16_logits: bool = True,
                         flags: int = 0, workspace: Optional[MoeWorkspace] = None) -> torch.Tensor:
     """``fused_experts(x, w1, w2, F.linear(x, gate_weight), ...)`` in one call: the whole MoE block of the model
     (models/mixtral.py:53-63) with the router gate computed inside the router's launch."""
@@ -204,8 +244,8 @@ def fused_experts_gated(hidden_states: torch.Tensor, gate_weight: torch.Tensor, 
         raise RuntimeError("the fused MoE path computes in bfloat16: hidden_states, gate_weight, w1 and w2 must be bfloat16")
     flags |= _w2_flag(w2)
     want_f32 = out_dtype == torch.float32
-    if accurate:
-        flags |= _lib.FLAG_ACCURATE
+    if bf16_act:
+        flags |= _lib.FLAG_BF16_ACT
     if not bf16_logits:
         flags |= _lib.FLAG_GATE_F32_LOGITS
     if want_f32 and inplace:
@@ -217,7 +257,7 @@ def fused_experts_gated(hidden_states: torch.Tensor, gate_weight: torch.Tensor, 
         output = hidden_states if inplace else torch.empty_like(hidden_states)
     if T == 0:
         return output
-    ws = workspace or get_workspace(hidden_states.device, T, H, I, E, topk)
+    ws = workspace or get_workspace(hidden_states.device, T, H, I, E, topk, flags)
     code = _lib.load().em_moe_forward_gated(
         hidden_states.data_ptr(), gate_weight.data_ptr(), w1.data_ptr(), w2.data_ptr(), output.data_ptr(),
         T, H, I, E, topk, 1 if renormalize else 0, ws.buffer.data_ptr(), ctypes.c_size_t(ws.buffer.numel()), flags,
@@ -274,7 +314,7 @@ def norm_gate_topk(hidden_states: torch.Tensor, residual: Optional[torch.Tensor]
 
 def fused_experts_normed(hidden_states: torch.Tensor, residual: Optional[torch.Tensor], norm_weight: torch.Tensor,
                          eps: float, gate_weight: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk: int,
-                         renormalize: bool = True, out_dtype: Optional[torch.dtype] = None, accurate: bool = False,
+                         renormalize: bool = True, out_dtype: Optional[torch.dtype] = None, bf16_act: bool = False,
                          bf16_logits: bool = True, op_rounding: bool = False, flags: int = 0,
                          workspace: Optional[MoeWorkspace] = None):
     """The tail of the reference's decoder layer in one call (models/mixtral.py:194-197):
@@ -289,8 +329,8 @@ def fused_experts_normed(hidden_states: torch.Tensor, residual: Optional[torch.T
     if w1.dtype != torch.bfloat16:
         raise RuntimeError("the fused MoE path computes in bfloat16: w1 and w2 must be bfloat16")
     flags |= _w2_flag(w2)
-    if accurate:
-        flags |= _lib.FLAG_ACCURATE
+    if bf16_act:
+        flags |= _lib.FLAG_BF16_ACT
     if not bf16_logits:
         flags |= _lib.FLAG_GATE_F32_LOGITS
     dev = hidden_states.device
@@ -303,7 +343,7 @@ def fused_experts_normed(hidden_states: torch.Tensor, residual: Optional[torch.T
         output = h_buf          # the experts' result overwrites the normalised rows, as the reference's in-place layer does
     if T == 0:
         return output, res_out
-    ws = workspace or get_workspace(dev, T, H, I, E, topk)
+    ws = workspace or get_workspace(dev, T, H, I, E, topk, flags)
     code = _lib.load().em_moe_forward_normed(
         hidden_states.data_ptr(), residual.data_ptr() if residual is not None else None, norm_weight.data_ptr(),
         _lib.dtype_code(norm_weight.dtype), float(eps), _lib.NORM_OP if op_rounding else _lib.NORM_LAYER,

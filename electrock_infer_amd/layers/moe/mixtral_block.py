@@ -39,20 +39,20 @@ class ReplicatedLinear(nn.Module):
 class MixtralMoE(nn.Module):
     """``forward(hidden_states)`` = ``experts(hidden_states, gate(hidden_states))`` of the reference
     (models/mixtral.py:53-63), with the gate computed inside the router's launch.  ``bf16_logits=True``
-    (default) rounds the logits to bf16 before the selection as the reference's bf16 gate does; ``accurate=True``
-    keeps the SiLU*mul activations as fp16 instead of bf16 through the w2 GEMM; ``w2_dtype=torch.float16`` keeps
-    ``experts.w2_weight`` as float16 (the loader's copy converts), which implies it at no cost in time."""
+    (default) rounds the logits to bf16 before the selection as the reference's bf16 gate does; ``bf16_act=True``
+    stores the SiLU*mul activations as bf16 instead of fp16 between the GEMMs; ``w2_dtype=torch.float16`` keeps
+    ``experts.w2_weight`` as float16 (the loader's copy converts), which saves the w2 GEMM its conversions."""
 
     def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int,
                  params_dtype: Optional[torch.dtype] = None, tp_size: Optional[int] = None, prefix: str = "",
-                 bf16_logits: bool = True, accurate: bool = False, w2_dtype: Optional[torch.dtype] = None):
+                 bf16_logits: bool = True, bf16_act: bool = False, w2_dtype: Optional[torch.dtype] = None):
         super().__init__()
         self.hidden_size = hidden_size
         self.bf16_logits = bf16_logits
         self.gate = ReplicatedLinear(hidden_size, num_experts, bias=False, params_dtype=params_dtype)
         self.experts = FusedMoE(num_experts=num_experts, top_k=top_k, hidden_size=hidden_size,
                                 intermediate_size=intermediate_size, params_dtype=params_dtype,
-                                reduce_results=True, renormalize=True, tp_size=tp_size, accurate=accurate,
+                                reduce_results=True, renormalize=True, tp_size=tp_size, bf16_act=bf16_act,
                                 w2_dtype=w2_dtype)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
@@ -61,7 +61,7 @@ class MixtralMoE(nn.Module):
         e = self.experts
         out = fused_experts_gated(hidden_states, self.gate.weight, e.w13_weight, e.w2_weight, topk=e.top_k,
                                   renormalize=e.renormalize, inplace=True, bf16_logits=self.bf16_logits,
-                                  accurate=e.accurate)
+                                  bf16_act=e.bf16_act)
         if e.reduce_results and e.tp_size > 1:
             dist.all_reduce(out)
         return out.view(orig_shape)
@@ -87,7 +87,7 @@ class PostAttentionMoE(nn.Module):
         orig_shape = hidden_states.shape
         out, res = fused_experts_normed(hidden_states.view(-1, moe.hidden_size), residual.view(-1, moe.hidden_size),
                                         norm.weight, norm.eps, moe.gate.weight, e.w13_weight, e.w2_weight, topk=e.top_k,
-                                        renormalize=e.renormalize, bf16_logits=moe.bf16_logits, accurate=e.accurate)
+                                        renormalize=e.renormalize, bf16_logits=moe.bf16_logits, bf16_act=e.bf16_act)
         if e.reduce_results and e.tp_size > 1:
             dist.all_reduce(out)
         return out.view(orig_shape), res.view(orig_shape)

@@ -42,14 +42,15 @@ extern "C" {
 #define EM_ERR_BUFFER_SIZE    (-6)
 #define EM_ERR_ALIGNMENT      (-7)
 
-/* em_moe_forward flags */
-#define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16      */
-#define EM_FLAG_ACCURATE       (1u << 1)  /* SiLU*mul activations kept beyond one bf16       */
-#define EM_FLAG_GATE_F32_LOGITS (1u << 2) /* em_moe_forward_gated: route on the fp32 logits,   */
-                                          /* not on their bf16 rounding                        */
-#define EM_FLAG_W2_F16         (1u << 3)  /* `w2` holds fp16 values; implies EM_FLAG_ACCURATE */
-#define EM_FLAG_WIDE_RANGE     (1u << 4)  /* bf16 output: w2 partial sums stay float32 at   */
-                                          /* every batch size (see em_moe_forward)          */
+/* em_moe_forward flags (0 = the defaults described at em_moe_forward) */
+#define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16                        */
+#define EM_FLAG_GATE_F32_LOGITS (1u << 2) /* em_moe_forward_gated: route on the fp32 logits,              */
+                                          /* not on their bf16 rounding                                   */
+#define EM_FLAG_W2_F16         (1u << 3)  /* `w2` holds fp16 values (converted once by the caller)        */
+#define EM_FLAG_BF16_ACT       (1u << 5)  /* SiLU*mul activations rounded to bf16 between the two GEMMs,  */
+                                          /* as the reference stores them (default: kept finer, see below) */
+#define EM_FLAG_F16_PARTIALS   (1u << 6)  /* bf16 output of large batches: w2 partial sums stored as fp16 */
+                                          /* (default: float32 at every batch size)                       */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
 #define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
 #define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
@@ -94,7 +95,7 @@ int em_topk_softmax(const void* logits, int logits_dtype, int64_t T, int E, int 
  *   logits_out    [T, E]  optional (may be NULL): the logits that were routed on, bf16 when
  *                         round_logits_bf16 != 0, float32 otherwise
  *   topk_weights  [T, k]  float32, topk_ids [T, k] int32, as em_topk_softmax
- * Limits: E in {8, 16}, H % 8 == 0, E * H * 2 <= 160 KiB (the gate matrix is kept in LDS).
+ * Limits: E in {8, 16}, H % 8 == 0 (the gate matrix is read from global memory: it stays in L2).
  */
 int em_gate_topk_softmax(const void* x, const void* gate_w, int64_t T, int H, int E, int k,
                          int renormalize, int round_logits_bf16, void* logits_out,
@@ -206,10 +207,13 @@ int em_add_rms_norm(const void* x_in, const void* residual_in, void* x_out, void
                     int semantics, void* stream);
 
 /*
- * Bytes of device workspace em_moe_forward needs for these shapes
- * (0 for invalid shapes).  The workspace must be 256-byte aligned.
+ * Bytes of device workspace em_moe_forward needs for these shapes and flags
+ * (0 for invalid shapes).  The workspace must be 256-byte aligned.  The size depends on
+ * EM_FLAG_BF16_ACT and EM_FLAG_FORCE_GENERIC only; pass the flags of the call.
+ * A larger buffer than asked for is always valid: a caller that serves many batch sizes can
+ * keep one workspace sized for its largest.
  */
-size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
+size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigned flags);
 
 /*
  * The whole layer:  out[t] = sum_j w[t,j] * W2[e_tj] ( silu(W1[e_tj] x_t) * (W3[e_tj] x_t) ).
@@ -223,28 +227,31 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k);
  *                             (mixtral_moe.py:64-70,137-143)
  *   w2            [E, H, I]   bf16 (mixtral_moe.py:75-79); fp16 with EM_FLAG_W2_F16
  *   out           [T, H]      bf16 (float32 with EM_FLAG_OUT_F32); may alias x
- *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k), 256-byte aligned
- * EM_FLAG_ACCURATE takes the one rounding to bf16 that the MFMA of the w2 GEMM
- * otherwise needs out of the result: the SiLU*mul activations are kept as fp16,
- * clamped to +-65504, and the w2 kernel converts its bf16 weight fragments to fp16
- * on the way to the MFMA.  Mean relative error 2e-4 instead of 1.7e-3; no cost in
- * time up to 64 tokens, 4-6 % above (at 8192 tokens: +10 % on the w2 GEMM).  For
- * shapes only the generic kernels take, the activations are kept as a bf16 pair
- * (value, rounding residual) and the residual is multiplied in a second pass over
- * w2.  Both forms meet max-abs 2e-2 / mean relative 1e-3 against the fp32 definition
- * with EM_FLAG_OUT_F32.
+ *   workspace     >= em_moe_workspace_bytes(T,H,I,E,top_k,flags), 256-byte aligned
+ * Arithmetic (flags = 0): bf16 operands, float32 accumulation in both GEMMs, SiLU*mul in
+ * float32, routing weight and top-k sum in float32, one rounding of the result to bf16.
+ * Between the GEMMs the activations are stored as fp16 (clamped to +-65504) and the w2
+ * GEMM runs on the fp16 MFMA with its bf16 weight fragments converted on the way (exactly,
+ * for every weight of magnitude 2^-14 .. 65504): mean relative error 2e-4 against the fp32
+ * definition, i.e. max-abs 2e-2 / mean relative 1e-3 are met with EM_FLAG_OUT_F32 (a bf16
+ * output adds its own rounding, 1.4e-3).  For shapes only the generic kernels take, the
+ * activations are kept as a bf16 pair (value, rounding residual) and the residual is
+ * multiplied in a second pass over w2, to the same bar.
+ * EM_FLAG_BF16_ACT stores the activations as bf16 instead, the reference's storage type
+ * (fused_moe.py:223-239: cache2), with its range and its rounding: mean relative error
+ * 1.7e-3; no conversions in the w2 GEMM (8192 tokens: -10 % on that kernel, no difference
+ * up to 64 tokens).
  * EM_FLAG_W2_F16: the caller keeps w2 as fp16 (converted once, e.g. when the weights
- * are loaded: exact for every bf16 weight of magnitude 2^-14 .. 65504).  The layer then
- * runs in accurate mode without the conversion: within 1-2 % of the default mode's time
- * at every batch size.  Only shapes the tuned kernels take; others return
- * EM_ERR_UNSUPPORTED.
- * Range: above 448 tokens with a bf16 output the partial sums of the w2 GEMM (one per
- * routed slot and K slice, before the routing weight) pass through fp16 and saturate at
- * +-65504, where the reference's bf16 pipeline does not.  EM_FLAG_WIDE_RANGE keeps them
- * float32 (T=8192: +1-2 % in time); a float32 output always does.
+ * are loaded).  Same results as the default without the conversion: within 1-2 % of
+ * EM_FLAG_BF16_ACT's time at every batch size.  Only shapes the tuned kernels take and not
+ * together with EM_FLAG_BF16_ACT; others return EM_ERR_UNSUPPORTED.
+ * EM_FLAG_F16_PARTIALS: above 448 tokens with a bf16 output the partial sums of the w2
+ * GEMM (one per routed slot and K slice, before the routing weight) are stored as fp16 and
+ * saturate at +-65504, where the reference's bf16 pipeline does not (T=8192: -1 to -2 % in
+ * time).  Ignored for other batch sizes and for a float32 output.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
- * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.
+ * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.  Unknown flag bits: EM_ERR_UNSUPPORTED.
  */
 int em_moe_forward(const void* x, const void* router_logits, int logits_dtype,
                    const void* w13, const void* w2, void* out,
@@ -274,13 +281,13 @@ typedef struct em_moe_layout {
     int64_t expert_ids_off, expert_ids_len;        /* [expert_ids_len] i32     */
     int64_t post_pad_off;                          /* [1] i32                  */
     int64_t seg_begin_off;                         /* [E+1] i32 padded segment starts */
-    int64_t act_off;                               /* [sorted_len, I] bf16 (fp16 in accurate mode) */
-    int64_t act_lo_off;                            /* [sorted_len, I] bf16, accurate mode of the generic kernels */
-    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 (fp16 above 448 tokens with a bf16 out) */
+    int64_t act_off;                               /* [sorted_len, I] fp16 (bf16 with EM_FLAG_BF16_ACT and in the generic kernels) */
+    int64_t act_lo_off;                            /* [sorted_len, I] bf16 rounding residuals of the generic kernels; -1: not reserved */
+    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 (fp16 with EM_FLAG_F16_PARTIALS) */
     int64_t total_bytes;
 } em_moe_layout;
 
-int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k,
+int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, unsigned flags,
                             em_moe_layout* layout);
 
 #ifdef __cplusplus

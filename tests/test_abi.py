@@ -62,16 +62,25 @@ def test_workspace_layout_is_consistent():
     for T, H, I in [(1, 4096, 14336), (64, 4096, 14336), (256, 4096, 14336), (8192, 4096, 14336),
                     (64, 256, 512), (4096, 6144, 16384)]:
         L = _lib.workspace_layout(T, H, I, 8, 2)
-        assert lib.em_moe_workspace_bytes(T, H, I, 8, 2) == L.total_bytes
+        assert lib.em_moe_workspace_bytes(T, H, I, 8, 2, 0) == L.total_bytes
         assert L.block_size == (16 if T <= 64 else 32)    # 32: the tiled kernel's fragment height
         assert L.sorted_len % L.block_size == 0 and L.sorted_len >= T * 2 + 8 * (L.block_size - 1)
         assert L.expert_ids_len * L.block_size == L.sorted_len
         offs = [L.topk_weights_off, L.topk_ids_off, L.sorted_ids_off, L.expert_ids_off, L.post_pad_off,
-                L.act_off, L.act_lo_off, L.y_off, L.total_bytes]
+                L.act_off, L.y_off, L.total_bytes]
         assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
-        assert L.act_lo_off - L.act_off >= L.sorted_len * I * 2 and L.y_off - L.act_lo_off >= L.sorted_len * I * 2
+        assert L.act_lo_off == -1                       # the tuned kernels keep no rounding residuals
+        assert L.y_off - L.act_off >= L.sorted_len * I * 2
         assert L.total_bytes - L.y_off >= L.ksplit * T * 2 * H * 4
-    assert lib.em_moe_workspace_bytes(4, 4097, 512, 8, 2) == 0
+        # the routing results sit at the same offsets whatever the flags; the generic kernels' default form adds act_lo
+        G = _lib.workspace_layout(T, H, I, 8, 2, _lib.FLAG_FORCE_GENERIC)
+        assert (G.topk_ids_off, G.sorted_ids_off, G.expert_ids_off, G.post_pad_off) == \
+               (L.topk_ids_off, L.sorted_ids_off, L.expert_ids_off, L.post_pad_off)
+        assert G.act_lo_off - G.act_off >= G.sorted_len * I * 2 and G.y_off - G.act_lo_off >= G.sorted_len * I * 2
+        B = _lib.workspace_layout(T, H, I, 8, 2, _lib.FLAG_FORCE_GENERIC | _lib.FLAG_BF16_ACT)
+        assert B.act_lo_off == -1 and B.total_bytes < G.total_bytes
+    assert lib.em_moe_workspace_bytes(4, 4097, 512, 8, 2, 0) == 0
+    assert lib.em_moe_workspace_bytes(4, 4096, 512, 8, 2, 1 << 30) == 0      # unknown flag bit
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -114,7 +114,7 @@ def test_mixtral_block_module():
 
 
 def test_mixtral_block_module_with_float16_w2():
-    """w2_dtype=float16 on the block: the same call as accurate mode on the bf16 weights, without the conversion."""
+    """w2_dtype=float16 on the block: the same call as the default mode on the bf16 weights, without the conversion."""
     from electrock_infer_amd import MixtralMoE
     from electrock_infer_amd.layers.moe.fused_moe import fused_experts_gated
     announce("MixtralMoE module, float16 w2")
@@ -128,7 +128,6 @@ def test_mixtral_block_module_with_float16_w2():
     for e in range(E):
         blk.experts.weight_loader(blk.experts.w2_weight, w2[e], "w2", e)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(DEV)
-    want = fused_experts_gated(x.clone(), blk.gate.weight, blk.experts.w13_weight, w2, topk=2, renormalize=True,
-                               accurate=True)
+    want = fused_experts_gated(x.clone(), blk.gate.weight, blk.experts.w13_weight, w2, topk=2, renormalize=True)
     got = blk(x.clone())
     assert float((got.float() - want.float()).abs().max()) <= 2.0 ** -8 * float(want.float().abs().max())

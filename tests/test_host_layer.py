@@ -27,9 +27,9 @@ def test_op_surface_matches_reference_binding():
         "num_experts", "top_k", "hidden_size", "intermediate_size", "tp_size", "params_dtype", "renormalize",
         "reduce_results"]
     # the additions are keyword-only and off by default
-    assert list(params)[9:] == ["accurate", "w2_dtype"]
-    assert all(params[k].kind is inspect.Parameter.KEYWORD_ONLY for k in ("accurate", "w2_dtype"))
-    assert params["accurate"].default is False and params["w2_dtype"].default is None
+    assert list(params)[9:] == ["bf16_act", "w2_dtype"]
+    assert all(params[k].kind is inspect.Parameter.KEYWORD_ONLY for k in ("bf16_act", "w2_dtype"))
+    assert params["bf16_act"].default is False and params["w2_dtype"].default is None
     assert em._C is _C
 
 
