@@ -64,3 +64,37 @@ def test_captured_decoder_tail_replays_bit_exact():
         assert torch.equal(out_g, out_e) and torch.equal(res_g, res_e), f"replay {rep}"
         fused_experts_normed(x, r, nw, 1e-5, gw, w13, w2, topk=2, workspace=ws)
         torch.cuda.synchronize()
+
+
+def test_graphs_of_two_batch_sizes_through_the_module_share_the_workspace():
+    """The usual capture pattern of an engine: eager warm-up and capture at one batch size, then at a larger one,
+    through FusedMoE.forward (which takes no workspace argument and uses the device's shared one).  The larger batch
+    makes the shared buffer grow; the first graph still holds the old address, so that buffer must stay alive: the
+    first graph, replayed after the second was captured and run, has to give its eager result -- also after other
+    allocations had the chance to land on freed memory."""
+    from electrock_infer_amd import FusedMoE
+    from electrock_infer_amd.layers.moe import fused_moe
+    announce("graph capture of two batch sizes through FusedMoE.forward")
+    H, I, E = 512, 1024, 8
+    fused_moe.release_workspaces(DEV)          # start from an empty cache so that the second size does grow it
+    x, lg, w13, w2 = gpu_inputs(96, H, I, E, seed=21)
+    layer = FusedMoE(E, 2, H, I, tp_size=1, params_dtype=torch.bfloat16).to(DEV)
+    layer.w13_weight.data, layer.w2_weight.data = w13, w2
+    graphs = []
+    for T in (8, 96):
+        xs, ls = x[:T].clone(), lg[:T].clone()
+        eager = layer(xs.clone(), ls).clone()
+        buf = xs.clone()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            out = layer(buf, ls)                # in place: out is buf
+        graphs.append((g, buf, xs, eager))
+    assert len(fused_moe._retired.get(torch.device(DEV).index, [])) >= 1     # the buffer did grow in between
+    junk = [torch.randn(1 << 20, device=DEV) for _ in range(8)]              # would reuse a freed workspace
+    for rep in range(2):
+        for g, buf, xs, eager in graphs:
+            buf.copy_(xs)
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(buf, eager), f"replay {rep}"
+    del junk
