@@ -27,12 +27,15 @@ FLAG_SKIP_GEMM2 = 1 << 11
 FLAG_SKIP_COMBINE = 1 << 12
 FLAG_FORCE_GENERIC = 1 << 16
 
+ERR_STATIC_LIMIT = -8
+STATIC_SCRATCH_BYTES = 32 << 20   # EM_STATIC_SCRATCH_BYTES
+
 # every symbol include/electrock_moe.h declares
 EXPORTED_SYMBOLS = (
     "em_version", "em_error_string", "em_topk_softmax", "em_moe_align_block_size",
     "em_silu_and_mul", "em_moe_sum", "em_moe_workspace_bytes", "em_moe_workspace_layout",
     "em_moe_forward", "em_moe_forward_gated", "em_gate_topk_softmax", "em_rms_norm", "em_add_rms_norm",
-    "em_norm_gate_topk_softmax", "em_moe_forward_normed",
+    "em_norm_gate_topk_softmax", "em_moe_forward_normed", "em_moe_forward_static",
 )
 
 
@@ -76,6 +79,8 @@ def load() -> ctypes.CDLL:
     lib.em_moe_workspace_layout.argtypes = [i64, i32, i32, i32, i32, u32, ctypes.POINTER(MoeLayout)]
     lib.em_moe_forward.restype = i32
     lib.em_moe_forward.argtypes = [vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
+    lib.em_moe_forward_static.restype = i32
+    lib.em_moe_forward_static.argtypes = [vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, u32, vp]
     lib.em_moe_forward_gated.restype = i32
     lib.em_moe_forward_gated.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, u32, vp]
     lib.em_gate_topk_softmax.restype = i32

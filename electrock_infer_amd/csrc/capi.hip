@@ -1,5 +1,7 @@
 // extern "C" surface of libelectrock_moe.so: argument checks, workspace layout
 // and stage sequencing.  No kernel code lives here.
+#include <atomic>
+
 #include "common.h"
 
 using namespace em;
@@ -144,6 +146,8 @@ const char* em_error_string(int code) {
         case EM_ERR_WORKSPACE: return "workspace too small";
         case EM_ERR_BUFFER_SIZE: return "output buffer too small";
         case EM_ERR_ALIGNMENT: return "pointer not sufficiently aligned";
+        case EM_ERR_STATIC_LIMIT:
+            return "shapes need more scratch memory than the fixed buffer of em_moe_forward_static (EM_STATIC_SCRATCH_BYTES)";
         default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
     }
 }
@@ -228,6 +232,29 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigne
 }  // extern "C"
 
 namespace {
+
+// Scratch memory of em_moe_forward_static: one array per GPU, held from the moment the library is loaded on a
+// device until the process ends.  In host code the name is only a handle for hipGetSymbolAddress; the device
+// address is looked up once per device and passed to the kernels like any caller-provided workspace.
+constexpr size_t kStaticScratchBytes = EM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticScratchBytes];
+
+int static_scratch(void** out) {
+    static std::atomic<void*> ptrs[64];
+    int dev = -1;
+    const hipError_t de = hipGetDevice(&dev);
+    if (de != hipSuccess) return static_cast<int>(de);
+    if (dev < 0 || dev >= 64) return EM_ERR_UNSUPPORTED;
+    void* ptr = ptrs[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {  // first call on this device (a race between threads at worst repeats the lookup)
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (ptr == nullptr || reinterpret_cast<uintptr_t>(ptr) % 256 != 0) return EM_ERR_ALIGNMENT;
+        ptrs[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return 0;
+}
 
 // RMSNorm in front of the block: x of the layer is then the buffer the normalised rows are written to
 struct NormFront {
@@ -375,6 +402,22 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype, c
                    void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
     return moe_forward_impl(x, router_logits, logits_dtype, nullptr, w13, w2, out, T, H, I, E, top_k, renormalize,
                             workspace, workspace_bytes, flags, stream);
+}
+
+int em_moe_forward_static(const void* x, const void* router_logits, int logits_dtype, const void* w13,
+                          const void* w2, void* out, int64_t T, int H, int I, int E, int top_k, int renormalize,
+                          unsigned flags, void* stream) {
+    if (!shapes_ok(T, H, I, E, top_k)) return EM_ERR_BAD_SHAPE;
+    if (flags & ~kKnownFlags) return EM_ERR_UNSUPPORTED;
+    em_moe_layout L;
+    const int rc = layout_from_plan(make_plan(T, H, I, E, top_k, flags), T, H, I, E, top_k, &L);
+    if (rc != 0) return rc;
+    if (static_cast<size_t>(L.total_bytes) > kStaticScratchBytes) return EM_ERR_STATIC_LIMIT;
+    void* ws = nullptr;
+    const int src = static_scratch(&ws);
+    if (src != 0) return src;
+    return moe_forward_impl(x, router_logits, logits_dtype, nullptr, w13, w2, out, T, H, I, E, top_k, renormalize, ws,
+                            kStaticScratchBytes, flags, stream);
 }
 
 int em_moe_forward_gated(const void* x, const void* gate_w, const void* w13, const void* w2, void* out,

@@ -5,8 +5,8 @@
  * Every entry point takes raw DEVICE pointers, plain sizes and a HIP stream
  * (passed as void* so that this header needs no HIP include), launches
  * asynchronously on that stream, never allocates, frees or retains memory and
- * keeps no state between calls (but a per-device note that a kernel attribute has
- * been set).  The caller guarantees that the device owning the pointers is current.
+ * keeps no state between calls (but per-device notes that a kernel attribute has
+ * been set and where em_moe_forward_static's scratch array lives).  The caller guarantees that the device owning the pointers is current.
  *
  * Return value of every function returning int:
  *     0   success (work is queued on `stream`)
@@ -41,6 +41,7 @@ extern "C" {
 #define EM_ERR_WORKSPACE      (-5)
 #define EM_ERR_BUFFER_SIZE    (-6)
 #define EM_ERR_ALIGNMENT      (-7)
+#define EM_ERR_STATIC_LIMIT   (-8)
 
 /* em_moe_forward flags (0 = the defaults described at em_moe_forward) */
 #define EM_FLAG_OUT_F32        (1u << 0)  /* `out` is float32 [T,H] instead of bf16                        */
@@ -258,6 +259,31 @@ int em_moe_forward(const void* x, const void* router_logits, int logits_dtype,
                    int64_t T, int H, int I, int E, int top_k, int renormalize,
                    void* workspace, size_t workspace_bytes, unsigned flags,
                    void* stream);
+
+/*
+ * em_moe_forward without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * scratch memory is a fixed array inside the library, EM_STATIC_SCRATCH_BYTES per GPU, held
+ * from the time the library is loaded until the process ends.  No counterpart in the
+ * reference, which allocates its intermediate tensors on every call (fused_moe.py:223-239).
+ * Arguments, flags, results and return codes as em_moe_forward; in addition
+ *   EM_ERR_STATIC_LIMIT  em_moe_workspace_bytes(T,H,I,E,top_k,flags) exceeds
+ *                        EM_STATIC_SCRATCH_BYTES (nothing is launched); the limit admits the
+ *                        decode batches of both Mixtral shapes (up to 64 tokens at 8x22B,
+ *                        about 190 at 8x7B).
+ * The call allocates and frees nothing.  Its first call on a device looks up the array's
+ * device address (hipGetSymbolAddress; the runtime may place the array in device memory only
+ * at that moment): make that call outside graph capture.
+ * All calls on one GPU share the one array, which keeps the last call's contents (the kernels
+ * write every element they read, nothing has to start at zero): calls that overlap on one GPU,
+ * on different streams or from different threads, race -- order them on one stream.
+ * The routing results are not readable through this entry point.
+ */
+#define EM_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int em_moe_forward_static(const void* x, const void* router_logits, int logits_dtype,
+                          const void* w13, const void* w2, void* out,
+                          int64_t T, int H, int I, int E, int top_k, int renormalize,
+                          unsigned flags, void* stream);
 
 /*
  * The same layer with the router gate inside: replaces MixtralMoE.forward
