@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=64, help="batch size T of the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end generation row")
+    ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the end-to-end model")
+    ap.add_argument("--e2e-requests", type=int, default=100, help="requests of the end-to-end run")
     ap.add_argument("--shape", choices=["8x7b", "8x22b"], default="8x7b",
                     help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
     ap.add_argument("--mode", choices=sorted(MODES), default="default_f32out",
@@ -298,6 +301,51 @@ def vendor_gemm(torch, dev, T, steps, warmup):
             "ms": ms, "tflops": 2.0 * M * N * K / ms / 1e9, "frac_of_peak": 2.0 * M * N * K / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS}
 
 
+def e2e_row(torch, layers, num_requests):
+    """The end-to-end configuration: a Mixtral-8x7B-shaped random-init bf16 model (GQA 32q/8kv heads, head_dim 128,
+    vocab 32000) generating for `num_requests` requests with prompts of 100-1024 uniform token ids and 100-256 output
+    tokens (ignore_eos, temperature 0.6) through the harness's scheduler and paged KV cache, as the reference's
+    bench.py:8-32 does.  Reports output tokens/s and the share of the GPU time spent in the MoE tail of the decoder
+    layers (post-attention norm + gate + router + experts), from HIP events around those calls."""
+    from random import Random
+    from electrock_infer_amd.harness import LLMEngine, ModelConfig, SamplingParams
+    rnd = Random(0)
+    t0 = time.perf_counter()
+    engine = LLMEngine(ModelConfig(num_hidden_layers=layers), max_model_len=4096, max_num_seqs=300,
+                       max_num_batched_tokens=32768, gpu_memory_utilization=0.90)
+    build_s = time.perf_counter() - t0
+    prompts = [[rnd.randrange(0, 32000) for _ in range(rnd.randint(100, 1024))] for _ in range(num_requests)]
+    sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=rnd.randint(100, 256)) for _ in range(num_requests)]
+    engine.generate([[rnd.randrange(0, 32000) for _ in range(40)]], SamplingParams(temperature=0.6, max_tokens=8, ignore_eos=True))
+    events = []
+    for layer in engine.model_runner.model.model.layers:
+        layer.moe_events = events
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    outs = engine.generate(prompts, sps)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    moe_ms = sum(a.elapsed_time(b) for a, b in events)
+    gpu_ms = start.elapsed_time(stop)
+    out_tokens = sum(len(o["token_ids"]) for o in outs)
+    st = engine.stats
+    row = {"row": "e2e", "layers": layers, "requests": num_requests, "prompt_tokens": sum(len(p) for p in prompts),
+           "output_tokens": out_tokens, "wall_s": wall, "output_tokens_per_s": out_tokens / wall,
+           "moe_share_of_gpu_time": moe_ms / gpu_ms, "moe_ms": moe_ms, "gpu_ms": gpu_ms,
+           "prefill_tokens_per_s": st["prefill_tokens"] / max(st["prefill_s"], 1e-9),
+           "decode_tokens_per_s": st["decode_tokens"] / max(st["decode_s"], 1e-9), "engine_stats": st,
+           "kv_blocks": engine.config.num_kvcache_blocks, "model_build_s": build_s,
+           "attention": "torch scaled_dot_product_attention over the gathered paged cache (harness, not the hot path)"}
+    del engine, events
+    from electrock_infer_amd.layers.moe.fused_moe import release_workspaces
+    release_workspaces()
+    torch.cuda.empty_cache()
+    return row
+
+
 def main():
     global H, I, OPERANDS
     args = parse_args()
@@ -362,6 +410,13 @@ def main():
         for mode in ("default", "bf16_act_f16_partials", "w2_f16_f32out"):
             table.append(measure(torch, big, w13, w2, 10, 3, mode=mode, host=err_host))
 
+    cpu = None if (args.no_cpu or host is None) else cpu_baseline(torch, T, w13, host)
+    if not args.no_e2e and not args.no_table and args.shape == "8x7b" and OPERANDS == "gaussian":
+        del w13, w2
+        LayerRunner.extra_weight_sets = []
+        torch.cuda.empty_cache()
+        table.append(e2e_row(torch, args.e2e_layers, args.e2e_requests))
+
     result = {
         "metric": f"Mixtral-{args.shape.upper().replace('X', 'x')} MoE layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms"],
@@ -374,7 +429,7 @@ def main():
                    "w2_dtype": "f16" if MODES[args.mode] & F_W2_F16 else "bf16", "weight_sets": args.weight_sets},
         "latency_us": head["latency_us"], "layer_hbm_gbs": head["hbm_gbs"], "layer_hbm_frac": head["hbm_frac"], "stage_ms": head["stage_ms"],
         "roofline": roofline,
-        "cpu_baseline": None if (args.no_cpu or host is None) else cpu_baseline(torch, T, w13, host),
+        "cpu_baseline": cpu,
         "table": table,
     }
     print(json.dumps(result))
