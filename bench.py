@@ -59,6 +59,8 @@ def parse_args():
                     help="8x7b: H=4096 I=14336 (the headline); 8x22b: H=6144 I=16384")
     ap.add_argument("--mode", choices=sorted(MODES), default="default_f32out",
                     help="flag set of the headline workload (see the module docstring)")
+    ap.add_argument("--extra-flags", type=lambda v: int(v, 0), default=0,
+                    help="diagnostic: flag bits OR-ed into every layer call (e.g. 0x20000 = EM_FLAG_NO_PERSIST)")
     ap.add_argument("--no-errors", action="store_true",
                     help="skip the error measurement against the fp32 oracle (it copies the weights to the host)")
     ap.add_argument("--weight-sets", type=int, default=1,
@@ -121,6 +123,7 @@ class LayerRunner:
     """Calls em_moe_forward through the C ABI with pre-allocated buffers."""
 
     extra_weight_sets = []      # [(w13, w2), ...] cycled through together with the set given to the constructor
+    extra_flags = 0             # diagnostic flag bits added to every call
 
     def __init__(self, torch, T, w13, w2, x, lg, mode_flags):
         import ctypes
@@ -146,7 +149,7 @@ class LayerRunner:
         code = self.lib.em_moe_forward(
             self.x.data_ptr(), self.lg.data_ptr(), self._lib.DTYPE_BF16, w13.data_ptr(), w2.data_ptr(),
             self.out.data_ptr(), self.T, H, I, E, TOPK, 1, self.ws.buffer.data_ptr(),
-            self.ctypes.c_size_t(self.ws.buffer.numel()), flags | self.mode_flags,
+            self.ctypes.c_size_t(self.ws.buffer.numel()), flags | self.mode_flags | LayerRunner.extra_flags,
             self.torch.cuda.current_stream().cuda_stream)
         self._lib.check(code, "em_moe_forward")
 
@@ -370,6 +373,7 @@ def main():
         print(json.dumps(vendor_gemm(torch, dev, args.tokens, min(args.steps, 30), min(args.warmup, 5))))
         return
     w13, w2 = make_weights(torch, dev)
+    LayerRunner.extra_flags = args.extra_flags
     LayerRunner.extra_weight_sets = [make_weights(torch, dev, seed=s) for s in range(1, args.weight_sets)]
     need_host = not (args.no_cpu and args.no_errors) and OPERANDS == "gaussian"
     host = HostWeights(w13, w2) if need_host else None

@@ -26,6 +26,7 @@ FLAG_SKIP_GEMM1 = 1 << 10
 FLAG_SKIP_GEMM2 = 1 << 11
 FLAG_SKIP_COMBINE = 1 << 12
 FLAG_FORCE_GENERIC = 1 << 16
+FLAG_NO_PERSIST = 1 << 17      # diagnostic: one workgroup per tile in the 256-row kernels
 
 ERR_STATIC_LIMIT = -8
 STATIC_SCRATCH_BYTES = 32 << 20   # EM_STATIC_SCRATCH_BYTES
@@ -43,7 +44,7 @@ class MoeLayout(ctypes.Structure):
     """Mirror of struct em_moe_layout."""
     _fields_ = [(n, ctypes.c_int64) for n in (
         "block_size", "topk_weights_off", "topk_ids_off", "sorted_ids_off", "sorted_len",
-        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "act_off", "act_lo_off", "y_off", "ksplit",
+        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "tickets_off", "act_off", "act_lo_off", "y_off", "ksplit",
         "total_bytes")]
 
 

@@ -64,7 +64,7 @@ bool shapes_ok(int64_t T, int H, int I, int E, int top_k) {
 
 constexpr unsigned kKnownFlags = EM_FLAG_OUT_F32 | EM_FLAG_GATE_F32_LOGITS | EM_FLAG_W2_F16 | EM_FLAG_BF16_ACT |
                                  EM_FLAG_F16_PARTIALS | EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN | EM_FLAG_SKIP_GEMM1 |
-                                 EM_FLAG_SKIP_GEMM2 | EM_FLAG_SKIP_COMBINE | EM_FLAG_FORCE_GENERIC;
+                                 EM_FLAG_SKIP_GEMM2 | EM_FLAG_SKIP_COMBINE | EM_FLAG_FORCE_GENERIC | EM_FLAG_NO_PERSIST;
 
 // What a layer call of these shapes and flags runs: which kernels, which storage types between them.  The
 // workspace layout and the stage sequencing both follow from it.
@@ -121,6 +121,7 @@ int layout_from_plan(const Plan& pl, int64_t T, int H, int I, int E, int top_k, 
     L->expert_ids_off = take(L->expert_ids_len * 4);
     L->post_pad_off = take(4);
     L->seg_begin_off = take((E + 1) * 4);
+    L->tickets_off = take(2 * 8 * 4);  // tile counters of the persistent w13 and w2 launches (one per XCD each)
     L->act_off = take(pl.sorted_len * static_cast<int64_t>(I) * 2);
     // the rounding residuals exist only where the shape-generic kernels run in the default (two-term) form
     L->act_lo_off = pl.act_pair ? take(pl.sorted_len * static_cast<int64_t>(I) * 2) : -1;
@@ -362,7 +363,8 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
         if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
-        return launch_gemm_tile(q, seg_begin, mode, s);
+        int* tickets = (flags & EM_FLAG_NO_PERSIST) ? nullptr : reinterpret_cast<int*>(ws + L.tickets_off) + (mode - 1) * 8;
+        return launch_gemm_tile(q, seg_begin, mode, tickets, s);
     };
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
         rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s)

@@ -196,7 +196,8 @@ int launch_gemm_stream(const MoeProblem& p, const int32_t* seg_begin, int mode, 
 bool tile_shape_ok(int H, int I);
 int tile_row_block();
 bool tile_supported(const MoeProblem& p);
-int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s);      // 256-row tiles
+int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, int* tickets /* 8 ints or null */,
+                     hipStream_t s);                                                               // 256-row tiles
 bool tile_mid_supported(const MoeProblem& p);                                                      // 64- / 128-row tiles
 int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile /* 64 | 128 */,
                          hipStream_t s);

@@ -69,24 +69,56 @@ constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, se
 // F16 (w2 GEMM in accurate mode): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
 // into fp16 once, before its first MFMA, and the fp16 MFMA of the same shape and rate runs instead.  F16 = 1 converts
 // bf16 weights, F16 = 2 takes weights that are fp16 in memory (MoeProblem::w2_f16) as they come.
-template <int MODE, bool STREAM, int F16>
+// PERSIST: the launch has one workgroup per CU (or fewer) and every workgroup walks tiles until none is left: its
+// first tile is the one its id names, the following ones come from a ticket counter per XCD (`tickets[8]`, zero
+// before the launch), so that tile i still runs on XCD i % 8 and tiles are handed out in the order above.  Nothing
+// but the ticket is shared between workgroups: a workgroup never waits for another one.
+template <int MODE, bool STREAM, int F16, bool PERSIST>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, const int32_t* __restrict__ seg_begin,
-                                                               int ntiles_n, int kslice) {
+                                                               int ntiles_n, int kslice, int ids_x, int nz,
+                                                               int* __restrict__ tickets) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     // ---- tile list: expert e owns ceil(rows_e / 256) row tiles ----
     int mtiles = 0;
     for (int e = 0; e < p.E; ++e) mtiles += (seg_begin[e + 1] - seg_begin[e] + kTM - 1) / kTM;
-    // ---- which tile.  Workgroup ids are dealt to the 8 XCDs round-robin by the hardware; XCD x takes the
-    // column tiles [x, x+1) * ntiles_n / 8 of every expert and walks them expert by expert, column by column,
-    // row tile fastest.  The CUs of an XCD then share a few weight tiles and all row tiles of the expert through
-    // their L2, every weight byte leaves HBM once, and the eight XCDs read the same token rows at the same time.
+    // Tile ids: [0, ids_x) for K slice 0, [ids_x, 2 * ids_x) for slice 1, ...; ids_x is a multiple of 8.
+    const int my_xcd = blockIdx.x % kXcds;
+    const int first_ticket = gridDim.x / kXcds;  // tiles 0 .. gridDim.x - 1 are the workgroups' first ones
+    int tile_n = blockIdx.x / kXcds;              // this XCD's tile_n-th tile comes next (PERSIST)
+    int next_n = -1;                              // thread 0: ticket drawn ahead, while the current tile runs
+    for (bool first_tile = true;; first_tile = false) {
+    int id_x, id_z;
+    if (PERSIST) {
+        if (!first_tile) {
+            // hand the next ticket to all waves through LDS (every byte of it belongs to the copy rings, which are
+            // idle between two tiles: the barriers fence the last reads of the tile before and the first copies of
+            // the next one)
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                if (next_n < 0) next_n = first_ticket + atomicAdd(&tickets[my_xcd], 1);
+                *reinterpret_cast<volatile int*>(smem) = next_n;
+                next_n = -1;
+            }
+            __syncthreads();
+            tile_n = __builtin_amdgcn_readfirstlane(*reinterpret_cast<volatile int*>(smem));
+            __syncthreads();
+        }
+        const int id = tile_n * kXcds + my_xcd;
+        if (tile_n >= (1 << 26) || id >= ids_x * nz) break;  // every wave of the workgroup leaves here together
+        id_z = id / ids_x;
+        id_x = id - id_z * ids_x;
+    } else {
+        if (!first_tile) break;
+        id_x = blockIdx.x;
+        id_z = blockIdx.y;
+    }
     int nt, mt, expert = 0;
     if (ntiles_n % kXcds == 0) {
         const int cols = ntiles_n / kXcds;
-        const int xcd = blockIdx.x % kXcds;
-        int local = blockIdx.x / kXcds;
-        if (local >= mtiles * cols) return;
+        const int xcd = id_x % kXcds;
+        int local = id_x / kXcds;
+        if (local >= mtiles * cols) { if (PERSIST) continue; return; }
         for (; expert < p.E - 1; ++expert) {
             const int t = ((seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM) * cols;
             if (local < t) break;
@@ -109,10 +141,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         // column count not divisible: contiguous ranges of 4 row tiles x all column tiles per XCD
         const int total = mtiles * ntiles_n;
         const int per_xcd = (total + kXcds - 1) / kXcds;
-        const int xcd = blockIdx.x % kXcds;
-        const int local = blockIdx.x / kXcds;
+        const int xcd = id_x % kXcds;
+        const int local = id_x / kXcds;
         const int logical = xcd * per_xcd + local;
-        if (local >= per_xcd || logical >= total) return;
+        if (local >= per_xcd || logical >= total) { if (PERSIST) continue; return; }
         const int group_sz = kGroupM * ntiles_n;
         const int group = logical / group_sz;
         const int in_group = logical - group * group_sz;
@@ -134,13 +166,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     const int64_t m0 = seg_begin[expert] + static_cast<int64_t>(mt * blk_base + (mt < blk_rem ? mt : blk_rem)) * kRowBlock;
     const int valid = (blk_base + (mt < blk_rem ? 1 : 0)) * kRowBlock;  // multiple of 32, >= 32
 
-    const int tid = threadIdx.x;
+    // (PERSIST: the thread index is made opaque once per tile, so that everything derived from it -- copy plans,
+    // operand offsets -- is worked out again for every tile instead of being kept in registers across the tile loop:
+    // the loop body needs all 256 registers a wave has here)
+    int tid_once = threadIdx.x;
+    if (PERSIST) asm volatile("" : "+v"(tid_once));
+    const int tid = tid_once;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 2;  // 0..1
     const int wn = wave & 3;   // 0..3
     const int K = (MODE == 1) ? p.H : p.I;
-    const int k_begin = blockIdx.y * kslice;
+    const int k_begin = id_z * kslice;
 
     // ---- copy plan: copy n of a stage lands at region n / 4, byte (n % 4) * 8 KB + wave * 1 KB + lane * 16.
     // Byte o of a region holds piece q ^ (u & 7) of 2-row group u = o / 256, q = (row & 1) * 8 + piece.
@@ -246,7 +283,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
 
     // Unit u = 0..3 of a K step: row half h = u & 1 (fragments 4h .. 4h+3), K half k32 = u >> 1.
     // Token fragments live in register set u & 1, weight fragments (shared by both row halves) in set k32.
+    // (defined values at the start of every tile: a wave with fewer than four blocks never reads the fragments it
+    // does not load, but the compiler cannot see that, and would carry all sixteen from one tile to the next)
     bf16x8_t fa[2][4], fb[2][4];
+    if (PERSIST) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                fa[i][j] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                fb[i][j] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+    }
     auto mma = [](const bf16x8_t& a, const bf16x8_t& b, f32x4_t c) {
         if (F16) {
             f16x8_t ha, hb;  // the registers already hold fp16 bits
@@ -323,6 +371,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     block_barrier();
     if (1 < nk) issue_a(1);
     if (2 < nk) issue_b(2, 2);
+    // the next tile's ticket is drawn now and looked at when this tile is done (the atomic counts as one more
+    // memory operation in flight for thread 0's wave, which can only make that wave's waits stricter)
+    if (PERSIST && threadIdx.x == 0) next_n = first_ticket + atomicAdd(&tickets[my_xcd], 1);
     int bs = 0;  // ring slot of the weight rows of step kt
     // The main loop for a wave with NMI = 1 .. 4 blocks of 32 rows (a compile-time constant: fixed instruction
     // mix).  After the barrier that ends step kt, the MFMAs of its last unit alternate with the copies of A(kt+2)
@@ -458,7 +509,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         uint8_t* ytile = smem + 1024 + wave * (32 * kPitchY);
         if (tid < kTM) slots[tid] = my_slot;
         __syncthreads();
-        const int64_t yoff = static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
+        const int64_t yoff = static_cast<int64_t>(id_z) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
         float* ybase = p.y + yoff;
         uint16_t* ybase_h = reinterpret_cast<uint16_t*>(p.y) + yoff;  // the same partial results as fp16 (p.y_f16)
 #pragma unroll
@@ -491,6 +542,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             __builtin_amdgcn_wave_barrier();
         }
     }
+    }  // next tile
 }
 
 }  // namespace
@@ -506,7 +558,15 @@ bool tile_supported(const MoeProblem& p) {
            int64_t{kTM} * p.I * 2 < lim;
 }
 
-int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hipStream_t s) {
+namespace {
+__global__ void zero_tickets_kernel(int* tickets) {
+    if (threadIdx.x < kXcds) tickets[threadIdx.x] = 0;
+}
+}  // namespace
+
+// tickets: kXcds ints of device memory of this launch's own (zeroed here, on the stream, right before the kernel);
+// nullptr: one workgroup per tile, handed out by the hardware.
+int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, int* tickets, hipStream_t s) {
     if (!tile_supported(p)) return EM_ERR_UNSUPPORTED;
     const int ntiles_n = (mode == 1) ? p.I / 128 : p.H / kTN;
     // upper bound of the sum over experts of ceil(padded rows_e / 256)
@@ -518,44 +578,68 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, hi
     // Opt in to more than 64 KB of dynamic LDS once per device.  The flags only cache an
     // idempotent runtime call; a race between threads at worst repeats it.
     static std::atomic<bool> attr_set[64];
+    static std::atomic<int> num_cus[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev].load(std::memory_order_acquire)) {
-        const void* kernels[8] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 0>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 1>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 1>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 2>),
-                                  reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 2>)};
+        const void* kernels[16] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 0, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 1, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 1, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 2, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 2, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 0, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 1, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 1, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 2, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 2, true>)};
         for (const void* k : kernels) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
             if (e != hipSuccess) return static_cast<int>(e);
         }
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < kXcds) cus = 256;
+        num_cus[dev].store(cus, std::memory_order_relaxed);
         attr_set[dev].store(true, std::memory_order_release);
     }
     // one row tile per expert on average up to 7/8 full: weights are read once -> streaming copies.  The w2 GEMM keeps
     // them up to 1.25 row tiles per expert (T=1024-1280: -7 % on the kernel); the w13 GEMM does not: its streaming form
     // also starts the tiles at different K offsets, which costs 8 % once most experts have two row tiles that share weights.
     const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * (mode == 1 ? 7 : 10);
-    const dim3 grid1(grid, 1), grid2(grid, static_cast<unsigned>(p.ksplit));
-    auto go = [&](auto kernel, dim3 g, int kslice) {
-        launch(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice);
-    };
-    if (mode == 1) {
-        if (stream_b) go(gemm_tile_kernel<1, true, 0>, grid1, p.H);
-        else go(gemm_tile_kernel<1, false, 0>, grid1, p.H);
-    } else if (p.act_f16 && p.w2_f16) {
-        if (stream_b) go(gemm_tile_kernel<2, true, 2>, grid2, p.I / p.ksplit);
-        else go(gemm_tile_kernel<2, false, 2>, grid2, p.I / p.ksplit);
-    } else if (p.act_f16) {
-        if (stream_b) go(gemm_tile_kernel<2, true, 1>, grid2, p.I / p.ksplit);
-        else go(gemm_tile_kernel<2, false, 1>, grid2, p.I / p.ksplit);
-    } else {
-        if (stream_b) go(gemm_tile_kernel<2, true, 0>, grid2, p.I / p.ksplit);
-        else go(gemm_tile_kernel<2, false, 0>, grid2, p.I / p.ksplit);
+    const int nz = (mode == 1) ? 1 : p.ksplit;
+    const int kslice = (mode == 1) ? p.H : p.I / p.ksplit;
+    const bool persist = tickets != nullptr;
+    dim3 g(grid, static_cast<unsigned>(nz));
+    if (persist) {
+        // one workgroup per CU (a workgroup takes all of a CU's LDS), a multiple of 8 so that ids map to XCDs
+        const int64_t ids = static_cast<int64_t>(grid) * nz;
+        const int64_t cus = num_cus[dev].load(std::memory_order_relaxed) / kXcds * kXcds;
+        g = dim3(static_cast<unsigned>(ids < cus ? ids : cus), 1);
+        launch(zero_tickets_kernel, dim3(1), dim3(64), 0, s, tickets);
     }
+    auto go = [&](auto kernel) {
+        launch(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice, static_cast<int>(grid), nz, tickets);
+    };
+#define EM_TILE_GO(MODE, F16)                                              \
+    do {                                                                   \
+        if (persist) {                                                     \
+            if (stream_b) go(gemm_tile_kernel<MODE, true, F16, true>);     \
+            else go(gemm_tile_kernel<MODE, false, F16, true>);             \
+        } else {                                                           \
+            if (stream_b) go(gemm_tile_kernel<MODE, true, F16, false>);    \
+            else go(gemm_tile_kernel<MODE, false, F16, false>);            \
+        }                                                                  \
+    } while (0)
+    if (mode == 1) EM_TILE_GO(1, 0);
+    else if (p.act_f16 && p.w2_f16) EM_TILE_GO(2, 2);
+    else if (p.act_f16) EM_TILE_GO(2, 1);
+    else EM_TILE_GO(2, 0);
+#undef EM_TILE_GO
     return launch_status();
 }
 

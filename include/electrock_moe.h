@@ -58,6 +58,8 @@ extern "C" {
 #define EM_FLAG_SKIP_GEMM2     (1u << 11)
 #define EM_FLAG_SKIP_COMBINE   (1u << 12)
 #define EM_FLAG_FORCE_GENERIC  (1u << 16) /* use the shape-generic GEMM kernels           */
+#define EM_FLAG_NO_PERSIST     (1u << 17) /* diagnostic: the 256-row kernels run one workgroup per tile  */
+                                          /* instead of one per CU walking a tile queue                  */
 
 /* Library version, e.g. 100 = 0.1.0. */
 int em_version(void);
@@ -307,6 +309,7 @@ typedef struct em_moe_layout {
     int64_t expert_ids_off, expert_ids_len;        /* [expert_ids_len] i32     */
     int64_t post_pad_off;                          /* [1] i32                  */
     int64_t seg_begin_off;                         /* [E+1] i32 padded segment starts */
+    int64_t tickets_off;                           /* [2][8] i32 tile counters of the large-batch GEMM launches */
     int64_t act_off;                               /* [sorted_len, I] fp16 (bf16 with EM_FLAG_BF16_ACT and in the generic kernels) */
     int64_t act_lo_off;                            /* [sorted_len, I] bf16 rounding residuals of the generic kernels; -1: not reserved */
     int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 (fp16 with EM_FLAG_F16_PARTIALS) */
