@@ -194,6 +194,29 @@ def test_layer_8x7b_prefill(mixtral_8x7b, logits):
     assert torch.allclose(out_p, out_def[perm], rtol=0, atol=1e-5)
 
 
+@pytest.mark.parametrize("T", [2048, 8192])
+def test_layer_8x7b_tuned_kernels_against_the_generic_kernels_on_every_row(mixtral_8x7b, T):
+    """The oracle checks a sample of the rows of the large batches; here every element of the tuned kernels' output is
+    compared with the shape-generic kernels' (another tiling, another copy path, no tile queue), which the oracle
+    checks in full on the small shapes of this file: a wrong tile at one (expert, row tile, column tile) cannot hide.
+    With bf16 activations both forms accumulate the same bf16 products in float32 through the same MFMA shape, K
+    ascending, over the same two K slices: the results are equal to the last bit (measured: difference 0.0).  In the
+    default form the tuned kernels keep the activations as fp16, the generic ones as a bf16 pair: 2^-12 apart."""
+    announce(f"layer 8x7B T={T}: tuned vs generic kernels, all rows")
+    m = mixtral_8x7b
+    x, lg = m["x"][:T].contiguous(), m["lg"][:T].contiguous()
+    for mode in (0, _lib.FLAG_BF16_ACT):
+        tuned = fused_experts(x, m["w13"], m["w2"], lg, 2, out_dtype=torch.float32, flags=mode)
+        generic = fused_experts(x, m["w13"], m["w2"], lg, 2, out_dtype=torch.float32, flags=mode | _lib.FLAG_FORCE_GENERIC)
+        d = (tuned - generic).abs()
+        scale = float(generic.abs().max())
+        tol = (1e-5 if mode else 1.5e-3) * scale          # measured: 0.0 and 2.0e-4 * scale
+        worst = float(d.max())
+        record(f"8x7b_T{T}_tuned_vs_generic_flags{mode}", max_abs=worst, scale=scale, mean_abs=float(d.mean()))
+        assert worst <= tol, (mode, worst, tol)
+        assert float(d.mean()) <= (1e-6 if mode else 8e-4) * float(generic.abs().mean())
+
+
 def test_layer_8x7b_float16_w2(mixtral_8x7b):
     """w2 handed over as float16 at the full 8x7B shape (decode, mid-size and prefill kernels): the stated target
     against the oracle on sampled tokens."""
