@@ -28,6 +28,10 @@ constexpr int64_t kStreamW2MaxT = 8;
 constexpr int64_t kTile64MaxT = 192;
 constexpr int64_t kTile128MaxT = 352;
 constexpr int64_t kTile128W2MaxT = 448;  // the w2 GEMM stays on 128-row tiles a little longer (156-160 against 165 us)
+// Up to this many tokens router and sort share one launch (a single workgroup, whose time grows with the batch);
+// above, the two kernels (the router on many workgroups) are faster than the launch they save (8x7B layer, fused
+// against separate: T=256 473.4 / 473.9 us, T=512 552.9 / 550.0, T=1024 929 / 920, T=2048 1428 / 1408).
+constexpr int64_t kFusedFrontMaxT = 256;
 
 // Rows per sorted block, the counterpart of _get_moe_config (fused_moe.py:327-339):
 // 16 (one MFMA fragment) for the streaming kernel, 32 for the tiled kernel, which cuts
@@ -336,7 +340,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.ksplit = static_cast<int>(L.ksplit);
 
     const bool fused_front = !(flags & (EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN)) && norm == nullptr &&
-                             gate_w == nullptr && route_align_supported(T, E, top_k);
+                             gate_w == nullptr && T <= kFusedFrontMaxT && route_align_supported(T, E, top_k);
     if (fused_front) {
         rc = launch_route_align(router_logits, logits_dtype, T, top_k, renormalize, topk_w, topk_ids, p.block, sorted,
                                 L.sorted_len, eids, L.expert_ids_len, post_pad, seg_begin, s);
