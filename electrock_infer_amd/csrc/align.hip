@@ -130,9 +130,11 @@ template <typename IdT, int EC>
 __global__ __launch_bounds__(kAlignThreads) void align_kernel(
     const IdT* __restrict__ ids, int64_t numel, int E_arg, int block,
     int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
-    int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out) {
+    int64_t eid_len, int32_t* __restrict__ post_pad, int32_t* __restrict__ seg_out,
+    int32_t* __restrict__ tickets /* 16 tile counters of the GEMM launches behind this sort to clear, or null */) {
     __shared__ int32_t hist[kAlignWaves][kMaxExperts];
     __shared__ int32_t seg_begin[kMaxExperts + 1];
+    if (tickets != nullptr && threadIdx.x < 16) tickets[threadIdx.x] = 0;
     align_body<IdT, EC>(ids, numel, E_arg, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out, hist,
                         seg_begin);
 }
@@ -175,18 +177,18 @@ __global__ __launch_bounds__(kAlignThreads) void route_align_kernel(
 
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
-                 int32_t* post_pad, int32_t* seg_out, hipStream_t s) {
+                 int32_t* post_pad, int32_t* seg_out, int32_t* tickets, hipStream_t s) {
     const dim3 grid(1), blk(kAlignThreads);
     if (itype == EM_ITYPE_I32) {
         if (E == 8)
             launch((align_kernel<int32_t, 8>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
-                               numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
+                               numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out, tickets);
         else
             launch((align_kernel<int32_t, 0>), grid, blk, 0, s, static_cast<const int32_t*>(ids),
-                               numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
+                               numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out, tickets);
     } else if (itype == EM_ITYPE_I64) {
         launch((align_kernel<int64_t, 0>), grid, blk, 0, s, static_cast<const int64_t*>(ids),
-                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out);
+                           numel, E, block, sorted, sorted_len, expert_ids, eid_len, post_pad, seg_out, tickets);
     } else {
         return EM_ERR_BAD_DTYPE;
     }

@@ -178,7 +178,7 @@ int em_moe_align_block_size(const void* topk_ids, int ids_itype, int64_t numel, 
         return EM_ERR_NULL_POINTER;
     if (sorted_len < 0 || expert_ids_len < 0) return EM_ERR_BUFFER_SIZE;
     return launch_align(topk_ids, ids_itype, numel, num_experts, block_size, sorted_token_ids, sorted_len,
-                        expert_ids, expert_ids_len, num_tokens_post_pad, nullptr, as_stream(stream));
+                        expert_ids, expert_ids_len, num_tokens_post_pad, nullptr, nullptr, as_stream(stream));
 }
 
 int em_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, void* stream) {
@@ -360,7 +360,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     }
     if (!fused_front && !(flags & EM_FLAG_SKIP_ALIGN)) {
         rc = launch_align(topk_ids, EM_ITYPE_I32, T * top_k, E, p.block, sorted, L.sorted_len, eids,
-                          L.expert_ids_len, post_pad, seg_begin, s);
+                          L.expert_ids_len, post_pad, seg_begin, reinterpret_cast<int32_t*>(ws + L.tickets_off), s);
         if (rc != 0) return rc;
     }
     const bool use_stream = pl.use_stream, use_tile = pl.use_tile;
@@ -368,7 +368,8 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
         if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
         int* tickets = (flags & EM_FLAG_NO_PERSIST) ? nullptr : reinterpret_cast<int*>(ws + L.tickets_off) + (mode - 1) * 8;
-        return launch_gemm_tile(q, seg_begin, mode, tickets, s);
+        // the sort kernel clears both launches' counters; a call that skips it (stage timing) clears them here
+        return launch_gemm_tile(q, seg_begin, mode, tickets, fused_front || (flags & EM_FLAG_SKIP_ALIGN) != 0, s);
     };
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
         rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s)

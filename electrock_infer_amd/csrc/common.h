@@ -144,6 +144,7 @@ int launch_norm_gate_router(const void* x_in, const void* res_in, const void* no
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
                  int32_t* post_pad, int32_t* seg_out /* [E+1] padded segment starts, may be null */,
+                 int32_t* tickets /* 16 tile counters to clear for the GEMM launches that follow, may be null */,
                  hipStream_t s);
 // Router + sort in one launch (eight experts, k * T slots within the kernel's LDS table).
 bool route_align_supported(int64_t T, int E, int k);
@@ -197,7 +198,7 @@ bool tile_shape_ok(int H, int I);
 int tile_row_block();
 bool tile_supported(const MoeProblem& p);
 int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, int* tickets /* 8 ints or null */,
-                     hipStream_t s);                                                               // 256-row tiles
+                     bool clear_tickets /* they were not cleared by the sort in front */, hipStream_t s);                                                               // 256-row tiles
 bool tile_mid_supported(const MoeProblem& p);                                                      // 64- / 128-row tiles
 int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile /* 64 | 128 */,
                          hipStream_t s);

@@ -564,9 +564,11 @@ __global__ void zero_tickets_kernel(int* tickets) {
 }
 }  // namespace
 
-// tickets: kXcds ints of device memory of this launch's own (zeroed here, on the stream, right before the kernel);
-// nullptr: one workgroup per tile, handed out by the hardware.
-int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, int* tickets, hipStream_t s) {
+// tickets: kXcds ints of device memory of this launch's own, zero when the kernel starts (cleared by the sort kernel in
+// front of the GEMMs, or here, on the stream, with clear_tickets); nullptr: one workgroup per tile, handed out by the
+// hardware.
+int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, int* tickets, bool clear_tickets,
+                     hipStream_t s) {
     if (!tile_supported(p)) return EM_ERR_UNSUPPORTED;
     const int ntiles_n = (mode == 1) ? p.I / 128 : p.H / kTN;
     // upper bound of the sum over experts of ceil(padded rows_e / 256)
@@ -620,7 +622,7 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
         const int64_t ids = static_cast<int64_t>(grid) * nz;
         const int64_t cus = num_cus[dev].load(std::memory_order_relaxed) / kXcds * kXcds;
         g = dim3(static_cast<unsigned>(ids < cus ? ids : cus), 1);
-        launch(zero_tickets_kernel, dim3(1), dim3(64), 0, s, tickets);
+        if (clear_tickets) launch(zero_tickets_kernel, dim3(1), dim3(64), 0, s, tickets);
     }
     auto go = [&](auto kernel) {
         launch(kernel, g, dim3(kThreads), lds_bytes, s, p, seg_begin, ntiles_n, kslice, static_cast<int>(grid), nz, tickets);
