@@ -19,6 +19,9 @@ errors of that very mode against the fp32 oracle on sampled tokens):
   bf16_act         EM_FLAG_BF16_ACT: activations stored as bf16 between the GEMMs (the reference's type)
   bf16_act_f16_partials  ... plus EM_FLAG_F16_PARTIALS: the fastest form for large batches
   w2_f16_f32out    EM_FLAG_W2_F16 | EM_FLAG_OUT_F32: w2 converted to fp16 once by the caller
+  f16_partials_f32out, w2_f16_f16_partials_f32out
+                   the two float32-output forms with EM_FLAG_F16_PARTIALS: w2 partial sums of large
+                   batches stored as fp16 (a caller's opt-in: they saturate at 65504)
 
 One JSON line is printed.  Besides the contract fields it carries
   roofline      the dominant kernel (w13 GEMM + SiLU*mul), timed alone with HIP
@@ -88,6 +91,8 @@ MODES = {
     "bf16_act": F_BF16_ACT,
     "bf16_act_f16_partials": F_BF16_ACT | F_F16_PARTIALS,
     "w2_f16_f32out": F_W2_F16 | F_OUT_F32,
+    "f16_partials_f32out": F_F16_PARTIALS | F_OUT_F32,
+    "w2_f16_f16_partials_f32out": F_W2_F16 | F_F16_PARTIALS | F_OUT_F32,
 }
 
 
@@ -411,7 +416,8 @@ def main():
         for mode in ("default", "bf16_act", "w2_f16_f32out"):
             if mode != args.mode:
                 table.append(measure(torch, T, w13, w2, half_steps, half_warm, mode=mode, host=err_host, stages=False))
-        for mode in ("default", "bf16_act_f16_partials", "w2_f16_f32out"):
+        for mode in ("default", "bf16_act_f16_partials", "w2_f16_f32out", "f16_partials_f32out",
+                     "w2_f16_f16_partials_f32out"):
             table.append(measure(torch, big, w13, w2, 10, 3, mode=mode, host=err_host))
 
     cpu = None if (args.no_cpu or host is None) else cpu_baseline(torch, T, w13, host)

@@ -19,7 +19,7 @@ FLAG_OUT_F32 = 1 << 0
 FLAG_GATE_F32_LOGITS = 1 << 2
 FLAG_W2_F16 = 1 << 3
 FLAG_BF16_ACT = 1 << 5        # SiLU*mul activations stored as bf16 between the GEMMs (the reference's storage type)
-FLAG_F16_PARTIALS = 1 << 6    # bf16 output of large batches: w2 partial sums stored as fp16
+FLAG_F16_PARTIALS = 1 << 6    # large batches: w2 partial sums stored as fp16
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10

@@ -104,7 +104,7 @@ Plan make_plan(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
     const bool bf16_act = (flags & EM_FLAG_BF16_ACT) != 0;
     pl.act_f16 = !bf16_act && (pl.use_stream || pl.use_tile);
     pl.act_pair = !bf16_act && !pl.act_f16;
-    pl.y_f16 = (flags & EM_FLAG_F16_PARTIALS) && !(flags & EM_FLAG_OUT_F32) && pl.use_tile && T > kTile128W2MaxT;
+    pl.y_f16 = (flags & EM_FLAG_F16_PARTIALS) && pl.use_tile && T > kTile128W2MaxT;
     return pl;
 }
 
@@ -313,8 +313,8 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.act_f16 = pl.act_f16 ? 1 : 0;
     p.w2_f16 = (flags & EM_FLAG_W2_F16) ? 1 : 0;
     // The partial results of the w2 GEMM (one per routed slot and K slice, before the routing weight) are float32.
-    // EM_FLAG_F16_PARTIALS stores those of the 256-row kernel as fp16 where the output is bf16 (their rounding, 2^-12,
-    // is far below the output's, 2^-9): half the bytes written by the kernel's epilogues, which all fall into the same
+    // EM_FLAG_F16_PARTIALS stores those of the 256-row kernel as fp16 (their rounding, 2^-12, is far below a bf16
+    // output's, 2^-9, and of the size of the fp16 activations'): half the bytes written by the kernel's epilogues, which all fall into the same
     // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer) -- but fp16 saturates
     // at 65504 where the reference's bf16 pipeline does not, so a caller has to ask for it.
     p.y_f16 = pl.y_f16 ? 1 : 0;

@@ -216,10 +216,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
     }
 }
 
-// The same sum over fp16 partial results, bf16 out: eight columns per thread (16-byte loads and stores).
-template <bool kStream>
+// The same sum over fp16 partial results: eight columns per thread (16-byte loads).
+template <bool kOutF32, bool kStream>
 __global__ __launch_bounds__(256) void combine_f16_kernel(const uint16_t* __restrict__ y, const float* __restrict__ w,
-                                                          uint16_t* __restrict__ out, int64_t T, int H, int top_k,
+                                                          void* __restrict__ out, int64_t T, int H, int top_k,
                                                           int ksplit) {
     const int64_t t = blockIdx.x;
     const int64_t zstride = T * top_k * static_cast<int64_t>(H);
@@ -241,9 +241,15 @@ __global__ __launch_bounds__(256) void combine_f16_kernel(const uint16_t* __rest
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[i] += wj * s[i];
         }
-        const u32x4_t o = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]),
-                           pack_bf16(acc[6], acc[7])};
-        *reinterpret_cast<u32x4_t*>(out + t * H + h) = o;
+        if (kOutF32) {
+            float* o = static_cast<float*>(out) + t * H + h;
+            *reinterpret_cast<f32x4_t*>(o) = f32x4_t{acc[0], acc[1], acc[2], acc[3]};
+            *reinterpret_cast<f32x4_t*>(o + 4) = f32x4_t{acc[4], acc[5], acc[6], acc[7]};
+        } else {
+            const u32x4_t o = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]),
+                               pack_bf16(acc[6], acc[7])};
+            *reinterpret_cast<u32x4_t*>(static_cast<uint16_t*>(out) + t * H + h) = o;
+        }
     }
 }
 
@@ -275,15 +281,16 @@ int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
     if (p.T == 0) return 0;
     // beyond the memory-side cache (256 MB) the partial results come back from HBM
     const bool stream = static_cast<int64_t>(p.ksplit) * p.T * p.top_k * p.H * (p.y_f16 ? 2 : 4) > (int64_t{256} << 20);
-    if (p.y_f16) {  // bf16 out only
-        if (out_f32 || p.H % 8 != 0) return EM_ERR_UNSUPPORTED;
+    if (p.y_f16) {
+        if (p.H % 8 != 0) return EM_ERR_UNSUPPORTED;
         const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 2048));
         const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
         auto go = [&](auto kernel) {
-            launch(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.topk_w,
-                               static_cast<uint16_t*>(out), p.T, p.H, p.top_k, p.ksplit);
+            launch(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.topk_w, out, p.T, p.H,
+                   p.top_k, p.ksplit);
         };
-        if (stream) go(combine_f16_kernel<true>); else go(combine_f16_kernel<false>);
+        if (out_f32) { if (stream) go(combine_f16_kernel<true, true>); else go(combine_f16_kernel<true, false>); }
+        else { if (stream) go(combine_f16_kernel<false, true>); else go(combine_f16_kernel<false, false>); }
         return launch_status();
     }
     const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 1024));

@@ -50,7 +50,7 @@ extern "C" {
 #define EM_FLAG_W2_F16         (1u << 3)  /* `w2` holds fp16 values (converted once by the caller)        */
 #define EM_FLAG_BF16_ACT       (1u << 5)  /* SiLU*mul activations rounded to bf16 between the two GEMMs,  */
                                           /* as the reference stores them (default: kept finer, see below) */
-#define EM_FLAG_F16_PARTIALS   (1u << 6)  /* bf16 output of large batches: w2 partial sums stored as fp16 */
+#define EM_FLAG_F16_PARTIALS   (1u << 6)  /* large batches: w2 partial sums stored as fp16 */
                                           /* (default: float32 at every batch size)                       */
 #define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
 #define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
@@ -248,10 +248,11 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigne
  * are loaded).  Same results as the default without the conversion: within 1-2 % of
  * EM_FLAG_BF16_ACT's time at every batch size.  Only shapes the tuned kernels take and not
  * together with EM_FLAG_BF16_ACT; others return EM_ERR_UNSUPPORTED.
- * EM_FLAG_F16_PARTIALS: above 448 tokens with a bf16 output the partial sums of the w2
- * GEMM (one per routed slot and K slice, before the routing weight) are stored as fp16 and
- * saturate at +-65504, where the reference's bf16 pipeline does not (T=8192: -1 to -2 % in
- * time).  Ignored for other batch sizes and for a float32 output.
+ * EM_FLAG_F16_PARTIALS: above 448 tokens the partial sums of the w2 GEMM (one per routed
+ * slot and K slice, before the routing weight) are stored as fp16 and saturate at +-65504,
+ * where the reference's bf16 pipeline does not (T=8192: -2 to -5 % in time; one more
+ * rounding of relative size 2^-12 per partial sum, mean relative error of a float32
+ * output 2.1e-4 -> 3e-4).  Ignored for smaller batches.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.  Unknown flag bits: EM_ERR_UNSUPPORTED.

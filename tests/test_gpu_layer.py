@@ -415,8 +415,8 @@ def test_default_mode_clamps_activations_at_the_fp16_range(T):
 
 def test_partial_sums_are_float32_unless_fp16_is_asked_for():
     """The partial sums of the w2 GEMM are float32 at every batch size, so the layer follows the definition at any
-    magnitude bf16 holds.  FLAG_F16_PARTIALS (a bf16 output above 448 tokens) stores them as fp16, which saturates at
-    65504: half the bytes, the caller's choice."""
+    magnitude bf16 holds.  FLAG_F16_PARTIALS (above 448 tokens) stores them as fp16, which saturates at 65504: half
+    the bytes, the caller's choice."""
     T = 600
     announce(f"output range, T={T}")
     x, lg, w13, w2 = mid_inputs(T, "normal", seed=31)
@@ -433,6 +433,9 @@ def test_partial_sums_are_float32_unless_fp16_is_asked_for():
         assert torch.isfinite(narrow).all()
         assert float(narrow.abs().max()) <= 4 * 65504 * 1.01        # two slots x two K slices, each saturated at most
         assert float((narrow - ref).abs().max()) > 0.1 * scale
+        narrow32 = fused_experts(xd, w13d, w2d, lgd, 2, out_dtype=torch.float32,
+                                 flags=mode | _lib.FLAG_F16_PARTIALS).cpu()
+        assert one_ulp_excess(narrow.to(torch.bfloat16), narrow32) == 0.0   # the same sums, rounded once more
 
 
 @pytest.mark.parametrize("T", [449, 777, 2100])
@@ -447,6 +450,14 @@ def test_fp16_partial_sums_within_their_rounding(T):
         half = fused_experts(x, w13, w2, lg, 2, flags=mode | _lib.FLAG_F16_PARTIALS)
         assert half.dtype == torch.bfloat16
         assert one_ulp_excess(half, f32) <= 2.0 ** -10 * float(f32.abs().max())
+        half32 = fused_experts(x, w13, w2, lg, 2, out_dtype=torch.float32, flags=mode | _lib.FLAG_F16_PARTIALS)
+        assert half32.dtype == torch.float32
+        assert float((half32 - f32).abs().max()) <= 2.0 ** -10 * float(f32.abs().max())
+        assert one_ulp_excess(half, half32) == 0.0
+        if mode == 0:   # the stated target holds with fp16 partial sums too
+            ref = O.moe_layer_fp32(*(t.cpu() for t in (x, lg, w13, w2)))
+            st = error_stats(half32.cpu(), ref)
+            assert st["max_abs"] <= 2e-2 and st["mean_rel"] <= 1e-3, st
 
 
 @pytest.mark.parametrize("T", [7, 64, 300, 777])
