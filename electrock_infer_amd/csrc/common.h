@@ -164,8 +164,8 @@ struct MoeProblem {
     const uint16_t* w13;      // [E, 2I, H] bf16
     const uint16_t* w2;       // [E, H, I] bf16 (fp16 when w2_f16)
     uint16_t* act;            // [sorted_len, I] bf16 (fp16 when act_f16), rows in sorted (padded) order
-    uint16_t* act_lo;         // same shape: bf16(value - act) in the accurate mode of the generic kernels, else null
-    int act_f16;              // act holds fp16 values (accurate mode of the tuned kernels; act_lo is null then)
+    uint16_t* act_lo;         // same shape: bf16(value - act) in the two-term form of the generic kernels, else null
+    int act_f16;              // act holds fp16 values (default form of the tuned kernels; act_lo is null then)
     int w2_f16;               // w2 holds fp16 values already: the fp16 w2 kernels skip their conversion
     int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
@@ -180,7 +180,7 @@ struct MoeProblem {
     int64_t sorted_len;       // worst-case padded length
     int ksplit;
 };
-// SiLU*mul result -> act (and the rounding residual -> act_lo in accurate mode)
+// SiLU*mul result -> act (and the rounding residual -> act_lo in the two-term form)
 __device__ __forceinline__ void store_act(const MoeProblem& p, int64_t idx, float v) {
     if (p.act_f16) {
         p.act[idx] = f32_to_f16_bits_sat(v);

@@ -15,7 +15,7 @@
 //   * the four partial accumulators meet once, at the end, in LDS.
 //
 //   MODE 1  64 rows = 32 gate rows j and the 32 up rows I + j of w13[e]; epilogue
-//           act[p, j] = silu(g) * u with g, u still in fp32, rounded once (bf16; fp16 in accurate mode)
+//           act[p, j] = silu(g) * u with g, u still in fp32, rounded once (fp16, or bf16 with EM_FLAG_BF16_ACT)
 //           (reference: Triton GEMM #1 + _C.silu_and_mul, fused_moe.py:250-272)
 //   MODE 2  64 rows n of w2[e], K slice z of I; epilogue y[z, slot, n] = partial sum
 //           (reference: Triton GEMM #2, fused_moe.py:282-287)
@@ -40,7 +40,7 @@ __device__ __forceinline__ u32x4_t ld16_stream(const uint16_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
 }
 
-// F16 (accurate mode, MODE 2 only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are turned
+// F16 (fp16 activations, MODE 2 only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are turned
 // into fp16 between the LDS tile and the MFMA (not when they are fp16 in memory, MoeProblem::w2_f16), which costs
 // this HBM-bound kernel nothing.
 template <int MODE, bool F16>

@@ -66,7 +66,7 @@ constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, se
 
 // STREAM: the weight rows are copied with the non-temporal hint.  Right when most experts fit one row tile
 // (every weight byte is then read by one workgroup only); wrong when several row tiles share them through L2.
-// F16 (w2 GEMM in accurate mode): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
+// F16 (w2 GEMM on fp16 activations): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
 // into fp16 once, before its first MFMA, and the fp16 MFMA of the same shape and rate runs instead.  F16 = 1 converts
 // bf16 weights, F16 = 2 takes weights that are fp16 in memory (MoeProblem::w2_f16) as they come.
 // PERSIST: the launch has one workgroup per CU (or fewer) and every workgroup walks tiles until none is left: its
