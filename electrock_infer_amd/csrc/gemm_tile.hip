@@ -114,7 +114,31 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         id_z = blockIdx.y;
     }
     int nt, mt, expert = 0;
-    if (ntiles_n % kXcds == 0) {
+    if (MODE == 2 && kXcds % nz == 0 && (ntiles_n * nz) % kXcds == 0) {
+        // w2 GEMM: an XCD works on one K slice only (slice xcd % nz), so its L2 fetches that slice of the activation
+        // rows instead of all of them, and on ntiles_n * nz / 8 of the column tiles of every expert
+        const int cols = ntiles_n * nz / kXcds;
+        const int xcd = id_x % kXcds;
+        int local = (id_z * ids_x + id_x) / kXcds;
+        if (local >= mtiles * cols) { if (PERSIST) continue; return; }
+        id_z = xcd % nz;
+        for (; expert < p.E - 1; ++expert) {
+            const int t = ((seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM) * cols;
+            if (local < t) break;
+            local -= t;
+        }
+        const int rows_e = (seg_begin[expert + 1] - seg_begin[expert] + kTM - 1) / kTM;
+        const int ngroups = (rows_e + kMaxGroupRows - 1) / kMaxGroupRows;
+        const int grows = (rows_e + ngroups - 1) / ngroups;
+        int g0 = 0, gr = grows;
+        for (;; g0 += grows) {
+            gr = (rows_e - g0 < grows) ? rows_e - g0 : grows;
+            if (local < gr * cols) break;
+            local -= gr * cols;
+        }
+        nt = (xcd / nz) * cols + local / gr;
+        mt = g0 + local % gr;
+    } else if (ntiles_n % kXcds == 0) {
         const int cols = ntiles_n / kXcds;
         const int xcd = id_x % kXcds;
         int local = id_x / kXcds;
