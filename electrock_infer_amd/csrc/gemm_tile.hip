@@ -402,13 +402,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     // The main loop for a wave with NMI = 1 .. 4 blocks of 32 rows (a compile-time constant: fixed instruction
     // mix).  After the barrier that ends step kt, the MFMAs of its last unit alternate with the copies of A(kt+2)
     // and B(kt+3) (the slots step kt has just freed) and with the first operand reads of step kt+1.
+    // w2 GEMM (kSpreadB): only the copies of A follow the barrier; the four of B(kt+3) are issued one step later,
+    // between the units of step kt+1.  All eight waves hand their copies to the address unit at the same moment, which
+    // works them off at one per 16 cycles: with half as many queued behind the barrier the activation rows, which
+    // have one step to arrive, are in LDS sooner (w2 kernel -2 % at 8192 tokens, -5 % at 1024), and the weight rows
+    // still have a step and a half.  The w13 GEMM is 1 % slower that way at 4096 tokens and more, and keeps its order.
+    // Either way the wait at the end of a step leaves exactly the newest four copies, B's, in flight.
+    constexpr bool kSpreadB = MODE == 2;
     auto main_loop = [&](auto nmi_tag) {
         constexpr int NMI = decltype(nmi_tag)::value;
         read_frags(0, 0, 0, nmi_tag);
         auto step = [&](int kt, auto copy_a_tag, auto copy_b_tag) {
             constexpr bool CA = decltype(copy_a_tag)::value, CB = decltype(copy_b_tag)::value;
+            // (kSpreadB: B(kt+2) goes to the slot that step kt-1 has freed, in between the units of this step)
+            const int bfree = bs == 0 ? kSlotsB - 1 : bs - 1;
+            if (kSpreadB && CB) { copy_b(0, kt + 2, bfree); copy_b(1, kt + 2, bfree); }
             read_frags(kt, bs, 1, nmi_tag); multiply(0, r4, nmi_tag);
+            if (kSpreadB && CB) copy_b(2, kt + 2, bfree);
             read_frags(kt, bs, 2, nmi_tag); multiply(1, r8, nmi_tag);
+            if (kSpreadB && CB) copy_b(3, kt + 2, bfree);
             read_frags(kt, bs, 3, nmi_tag); multiply(2, r4, nmi_tag);
             if (CA) wait_dma<kDmaHalf>(); else wait_dma<0>();   // this wave's parts of A(kt+1), B(kt+1) are in LDS
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // its last reads of step kt are in registers
@@ -427,7 +439,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     acc[4 + j][g] = mma(fa[1][j], fb[1][g], acc[4 + j][g]);
                 const int n = i >> 1;
                 if ((i & 1) == 0) {
-                    if (n < 4) { if (CA && (NMI == 4 || live[n])) copy_a(n, kt + 2); } else { if (CB) copy_b(n - 4, kt + 3, bs); }
+                    if (n < 4) { if (CA && (NMI == 4 || live[n])) copy_a(n, kt + 2); }
+                    else { if (!kSpreadB && CB) copy_b(n - 4, kt + 3, bs); }
                 } else if (n == 0) {
                     fb[0][0] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0]);
                 } else if (n == 1) {
@@ -442,8 +455,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             bs = bn;
         };
         int kt = 0;
-        for (; kt + 3 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
-        for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::false_type{});
+        if (kSpreadB) {
+            // step kt requests B(kt+2) while it multiplies (the prologue requested B(2)) and A(kt+2) behind its barrier
+            if (kt + 2 < nk) { step(kt, std::true_type{}, std::false_type{}); ++kt; }
+            for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
+        } else {
+            for (; kt + 3 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
+            for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::false_type{});
+        }
         for (; kt + 1 < nk; ++kt) step(kt, std::false_type{}, std::false_type{});
         read_frags(nk - 1, bs, 1, nmi_tag); multiply(0, r4, nmi_tag);
         read_frags(nk - 1, bs, 2, nmi_tag); multiply(1, r8, nmi_tag);
