@@ -607,6 +607,30 @@ def test_layer_drawn_shapes(seed):
     assert sb["mean_rel"] <= TOL_MEAN_REL_BF16, sb
 
 
+@pytest.mark.parametrize("I", [128, 256, 384, 512, 640])
+@pytest.mark.parametrize("T", [500, 1300])
+def test_layer_256_row_kernel_with_short_reductions(T, I):
+    """The 256-row kernels request their operands one to three K steps ahead; with I / 2 = 64 ... 320 the w2 GEMM has
+    one to five K steps per slice (H = 256: four for the w13 GEMM), which walks the first and last steps of the copy
+    schedule without the steady state in between, in every flag combination that changes that schedule."""
+    announce(f"256-row kernel, short reductions: T={T} H=256 I={I}")
+    x, lg, w13, w2 = O.make_inputs(T, 256, I, seed=T + I, logits="zipf")
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    outs = {}
+    for name, flags in (("default", 0), ("no_queue", _lib.FLAG_NO_PERSIST), ("bf16_act", _lib.FLAG_BF16_ACT)):
+        outs[name] = fused_experts(xd, w13d, w2d, lgd, 2, out_dtype=torch.float32, flags=flags)
+    outs["w2_f16"] = fused_experts(xd, w13d, w2d.to(torch.float16), lgd, 2, out_dtype=torch.float32)
+    check_routing(get_workspace(DEV, T, 256, I, 8, 2), lg.float(), T)
+    for name, out in outs.items():
+        st = error_stats(out.cpu(), ref)
+        if name == "bf16_act":
+            assert st["mean_rel"] <= TOL_MEAN_REL_F32 and st["max_abs"] <= TOL_MAX_ABS_F32 * float(ref.abs().max()), (name, st)
+        else:
+            assert st["max_abs"] <= TARGET_MAX_ABS and st["mean_rel"] <= TARGET_MEAN_REL, (name, st)
+    assert torch.equal(outs["default"], outs["no_queue"])
+
+
 def test_layer_shape_only_the_generic_kernel_supports():
     """H and I that are multiples of 8 but fit neither tuned kernel."""
     announce("layer odd shape H=136 I=200")
