@@ -80,7 +80,7 @@ struct Plan {
     bool w2_on_mid;             // streaming-size batch whose w2 GEMM runs on the 64-row tiled kernel
     bool act_f16;               // SiLU*mul activations stored as fp16 (tuned kernels, default)
     bool act_pair;              // ... as a bf16 pair (value, rounding residual): generic kernels, default
-    bool y_f16;                 // w2 partial sums stored as fp16 (opt-in, 256-row kernel, bf16 output)
+    bool y_f16;                 // w2 partial sums stored as fp16 (opt-in, 256-row kernel)
 };
 
 Plan make_plan(int64_t T, int H, int I, int E, int top_k, unsigned flags) {

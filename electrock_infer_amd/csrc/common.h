@@ -169,7 +169,7 @@ struct MoeProblem {
     int w2_f16;               // w2 holds fp16 values already: the fp16 w2 kernels skip their conversion
     int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
-    int y_f16;                // y holds fp16 values instead (256-row kernel with a bf16 layer output)
+    int y_f16;                // y holds fp16 values instead (256-row kernel, EM_FLAG_F16_PARTIALS)
     const int32_t* sorted_ids;
     const int32_t* expert_ids;
     const int32_t* post_pad;

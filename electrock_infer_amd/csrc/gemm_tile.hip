@@ -17,10 +17,10 @@
 //              between; eight lanes fetch one full 128-byte line of a row (measured
 //              L2 -> CU feed: ~26 TB/s with 128 B per row against ~17 TB/s with 64 B).
 //              Weight rows stream from HBM and are requested two K steps before their
-//              use, token rows (L2 / memory-side cache hits) one step before; with a
-//              single stage in flight the slowest line of a stage, at HBM latency, sat
-//              on the critical path of every step.  Completion is tracked by hand with
-//              s_waitcnt vmcnt + one s_barrier per step.
+//              use (w2 GEMM: one and a half, see the main loop), token rows (L2 / memory-side
+//              cache hits) one step before; with a single stage in flight the slowest line of
+//              a stage, at HBM latency, sat on the critical path of every step.  Completion is
+//              tracked by hand with s_waitcnt vmcnt + one s_barrier per step.
 //   issue      the eight copy instructions of a wave are issued one by one between the
 //              MFMAs that follow the barrier: issued back to back (by both waves of
 //              a SIMD at once) they left the matrix pipe idle for a fifth of every step
@@ -41,7 +41,9 @@
 //   order      workgroup ids are dealt to the 8 XCDs round-robin by the hardware; each XCD
 //              takes an eighth of the column tiles of every expert and walks them expert by
 //              expert, column by column, row tile fastest, so that the 32 CUs of an XCD share
-//              weight and token tiles through their own L2 and weights leave HBM once.
+//              weight and token tiles through their own L2 and weights leave HBM once.  In the
+//              w2 GEMM an XCD also stays on one K slice, so it fetches that slice of the
+//              activation rows only.
 #include <atomic>
 
 #include "common.h"
