@@ -314,9 +314,10 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.w2_f16 = (flags & EM_FLAG_W2_F16) ? 1 : 0;
     // The partial results of the w2 GEMM (one per routed slot and K slice, before the routing weight) are float32.
     // EM_FLAG_F16_PARTIALS stores those of the 256-row kernel as fp16 (their rounding, 2^-12, is far below a bf16
-    // output's, 2^-9, and of the size of the fp16 activations'): half the bytes written by the kernel's epilogues, which all fall into the same
-    // moments of a launch, and half the bytes read by the combine (T=8192: -2.5 % of the layer) -- but fp16 saturates
-    // at 65504 where the reference's bf16 pipeline does not, so a caller has to ask for it.
+    // output's, 2^-9, and of the size of the fp16 activations'): half the bytes written by the kernel's epilogues,
+    // which all fall into the same moments of a launch, and half the bytes read by the combine (T=8192: -1 to -2.5 %
+    // of the layer) -- but fp16 saturates at 65504 where the reference's bf16 pipeline does not, so a caller has to
+    // ask for it.
     p.y_f16 = pl.y_f16 ? 1 : 0;
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
