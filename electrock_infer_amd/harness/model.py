@@ -29,6 +29,7 @@ class BatchContext:
     block_tables: Optional[torch.Tensor] = None      # [seqs, max_blocks] int64, padded with 0
     context_lens: Optional[torch.Tensor] = None      # decode: [seqs] int64
     last_token_index: Optional[torch.Tensor] = None  # prefill: row of every sequence's last token
+    decode_mask: Optional[torch.Tensor] = None       # decode: [seqs, 1, 1, max_blocks * block_size] bool, key < context length
 
 
 class RotaryEmbedding(nn.Module):
@@ -59,6 +60,7 @@ class PagedAttention(nn.Module):
         self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
         self.scale = head_dim ** -0.5
         self.k_cache = self.v_cache = None            # [blocks, block_size, kv_heads, head_dim], set by the runner
+        self.kv_cache = None                          # the two as one tensor [2, blocks, block_size, kv_heads, head_dim]
 
     def _gathered(self, cache: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
         """[seqs, max_blocks * block_size, kv_heads, head_dim] from block ids [seqs, max_blocks]"""
@@ -75,12 +77,10 @@ class PagedAttention(nn.Module):
             # One new token per sequence: the query heads that share a KV head are laid out as the rows of one
             # small attention problem per (sequence, KV head), so the gathered keys are used as they are.
             B, group = q.shape[0], self.num_heads // self.num_kv_heads
-            keys = self._gathered(self.k_cache, ctx.block_tables).transpose(1, 2)     # [B, kvh, L, d]
-            vals = self._gathered(self.v_cache, ctx.block_tables).transpose(1, 2)
-            L = keys.shape[2]
-            mask = (torch.arange(L, device=q.device)[None, :] < ctx.context_lens[:, None])[:, None, None, :]
-            o = F.scaled_dot_product_attention(q.view(B, self.num_kv_heads, group, self.head_dim), keys, vals,
-                                               attn_mask=mask, scale=self.scale)
+            # keys and values of all sequences in one gather: [2, B, L, kvh, d] -> [B, kvh, L, d] each
+            kv = self.kv_cache[:, ctx.block_tables].view(2, B, -1, self.num_kv_heads, self.head_dim).transpose(2, 3)
+            o = F.scaled_dot_product_attention(q.view(B, self.num_kv_heads, group, self.head_dim), kv[0], kv[1],
+                                               attn_mask=ctx.decode_mask, scale=self.scale)
             return o.reshape(B, self.num_heads * self.head_dim)
         out = torch.empty_like(q)
         row = 0

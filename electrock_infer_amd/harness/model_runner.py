@@ -47,6 +47,7 @@ class ModelRunner:
         for i, layer in enumerate(self.model.model.layers):
             layer.self_attn.attn.k_cache = self.kv_cache[0, i]
             layer.self_attn.attn.v_cache = self.kv_cache[1, i]
+            layer.self_attn.attn.kv_cache = self.kv_cache[:, i]
 
     # ---- batch preparation ----
     def _to_device(self, values, dtype) -> torch.Tensor:
@@ -83,6 +84,9 @@ class ModelRunner:
         slots = [s.block_table[-1] * self.block_size + s.last_block_num_tokens - 1 for s in seqs]
         ctx = BatchContext(False, self._to_device(slots, torch.int64), [], [], block_tables=self._block_tables(seqs),
                            context_lens=self._to_device([len(s) for s in seqs], torch.int64))
+        # the same for every layer of the step: key j of a sequence counts if j < its context length
+        keys = ctx.block_tables.shape[1] * self.block_size
+        ctx.decode_mask = (torch.arange(keys, device=self.device)[None, :] < ctx.context_lens[:, None])[:, None, None, :]
         return self._to_device(input_ids, torch.int64), self._to_device(positions, torch.int64), ctx
 
     # ---- one step ----
