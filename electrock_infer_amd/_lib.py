@@ -20,13 +20,15 @@ FLAG_GATE_F32_LOGITS = 1 << 2
 FLAG_W2_F16 = 1 << 3
 FLAG_BF16_ACT = 1 << 5        # SiLU*mul activations stored as bf16 between the GEMMs (the reference's storage type)
 FLAG_F16_PARTIALS = 1 << 6    # large batches: w2 partial sums stored as fp16
+# diagnostic switches (include/electrock_moe_diag.h): benchmarks and tests only
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
 FLAG_SKIP_GEMM1 = 1 << 10
 FLAG_SKIP_GEMM2 = 1 << 11
 FLAG_SKIP_COMBINE = 1 << 12
 FLAG_FORCE_GENERIC = 1 << 16
-FLAG_NO_PERSIST = 1 << 17      # diagnostic: one workgroup per tile in the 256-row kernels
+FLAG_NO_PERSIST = 1 << 17      # one workgroup per tile in the 256-row kernels
+FLAG_ONE_GROUP_SORT = 1 << 18  # the layer's sort on one workgroup at every batch size
 
 ERR_STATIC_LIMIT = -8
 STATIC_SCRATCH_BYTES = 32 << 20   # EM_STATIC_SCRATCH_BYTES
@@ -36,7 +38,7 @@ EXPORTED_SYMBOLS = (
     "em_version", "em_error_string", "em_topk_softmax", "em_moe_align_block_size",
     "em_silu_and_mul", "em_moe_sum", "em_moe_workspace_bytes", "em_moe_workspace_layout",
     "em_moe_forward", "em_moe_forward_gated", "em_gate_topk_softmax", "em_rms_norm", "em_add_rms_norm",
-    "em_norm_gate_topk_softmax", "em_moe_forward_normed", "em_moe_forward_static",
+    "em_norm_gate_topk_softmax", "em_moe_forward_normed", "em_moe_forward_static", "em_moe_w2_f16_max_tokens",
 )
 
 
@@ -44,7 +46,8 @@ class MoeLayout(ctypes.Structure):
     """Mirror of struct em_moe_layout."""
     _fields_ = [(n, ctypes.c_int64) for n in (
         "block_size", "topk_weights_off", "topk_ids_off", "sorted_ids_off", "sorted_len",
-        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "tickets_off", "act_off", "act_lo_off", "y_off", "ksplit",
+        "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "tickets_off", "saturated_off",
+        "sort_scratch_off", "act_off", "act_lo_off", "y_off", "ksplit",
         "total_bytes")]
 
 
@@ -74,6 +77,8 @@ def load() -> ctypes.CDLL:
     lib.em_silu_and_mul.argtypes = [vp, vp, i64, i64, i32, vp]
     lib.em_moe_sum.restype = i32
     lib.em_moe_sum.argtypes = [vp, vp, i64, i32, i64, i32, vp]
+    lib.em_moe_w2_f16_max_tokens.restype = i64
+    lib.em_moe_w2_f16_max_tokens.argtypes = [i32, i32, i32, i32]
     lib.em_moe_workspace_bytes.restype = sz
     lib.em_moe_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, u32]
     lib.em_moe_workspace_layout.restype = i32

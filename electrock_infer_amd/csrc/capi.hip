@@ -3,12 +3,13 @@
 #include <atomic>
 
 #include "common.h"
+#include "../../include/electrock_moe_diag.h"
 
 using namespace em;
 
 namespace {
 
-constexpr int kVersion = 200;
+constexpr int kVersion = 300;
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 inline bool dtype_ok(int d) { return d == EM_DTYPE_F32 || d == EM_DTYPE_BF16 || d == EM_DTYPE_F16; }
@@ -32,6 +33,10 @@ constexpr int64_t kTile128W2MaxT = 448;  // the w2 GEMM stays on 128-row tiles a
 // above, the two kernels (the router on many workgroups) are faster than the launch they save (8x7B layer, fused
 // against separate: T=256 473.4 / 473.9 us, T=512 552.9 / 550.0, T=1024 929 / 920, T=2048 1428 / 1408).
 constexpr int64_t kFusedFrontMaxT = 256;
+// From this many routed slots (T * top_k) the sort of a layer call runs on several workgroups (two launches whose
+// histogram lives in the workspace); below, the one-workgroup kernel is as fast and one launch (timed alone, one
+// workgroup / several: 4096 slots 7.7 / 10.3 us, 16384 slots 18.5 / 10.7 us, 65536 slots 62 / 12 us).
+constexpr int64_t kMultiSortMinSlots = 8192;
 
 // Rows per sorted block, the counterpart of _get_moe_config (fused_moe.py:327-339):
 // 16 (one MFMA fragment) for the streaming kernel, 32 for the tiled kernel, which cuts
@@ -68,7 +73,8 @@ bool shapes_ok(int64_t T, int H, int I, int E, int top_k) {
 
 constexpr unsigned kKnownFlags = EM_FLAG_OUT_F32 | EM_FLAG_GATE_F32_LOGITS | EM_FLAG_W2_F16 | EM_FLAG_BF16_ACT |
                                  EM_FLAG_F16_PARTIALS | EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN | EM_FLAG_SKIP_GEMM1 |
-                                 EM_FLAG_SKIP_GEMM2 | EM_FLAG_SKIP_COMBINE | EM_FLAG_FORCE_GENERIC | EM_FLAG_NO_PERSIST;
+                                 EM_FLAG_SKIP_GEMM2 | EM_FLAG_SKIP_COMBINE | EM_FLAG_FORCE_GENERIC | EM_FLAG_NO_PERSIST |
+                                 EM_FLAG_ONE_GROUP_SORT;
 
 // What a layer call of these shapes and flags runs: which kernels, which storage types between them.  The
 // workspace layout and the stage sequencing both follow from it.
@@ -125,7 +131,11 @@ int layout_from_plan(const Plan& pl, int64_t T, int H, int I, int E, int top_k, 
     L->expert_ids_off = take(L->expert_ids_len * 4);
     L->post_pad_off = take(4);
     L->seg_begin_off = take((E + 1) * 4);
-    L->tickets_off = take(2 * 8 * 4);  // tile counters of the persistent w13 and w2 launches (one per XCD each)
+    // the call's counters, cleared by the sort: tile tickets of the persistent w13 and w2 launches (one per XCD
+    // each), then the count of clamped activations
+    L->tickets_off = take(32 * 4);
+    L->saturated_off = L->tickets_off + kSaturatedCounter * 4;
+    L->sort_scratch_off = take(align_scratch_ints(slots, E) * 4);
     L->act_off = take(pl.sorted_len * static_cast<int64_t>(I) * 2);
     // the rounding residuals exist only where the shape-generic kernels run in the default (two-term) form
     L->act_lo_off = pl.act_pair ? take(pl.sorted_len * static_cast<int64_t>(I) * 2) : -1;
@@ -228,6 +238,19 @@ int em_moe_workspace_layout(int64_t T, int H, int I, int E, int top_k, unsigned 
     return layout_from_plan(make_plan(T, H, I, E, top_k, flags), T, H, I, E, top_k, L);
 }
 
+int64_t em_moe_w2_f16_max_tokens(int H, int I, int E, int top_k) {
+    if (!shapes_ok(1, H, I, E, top_k)) return 0;
+    // every batch size must land on kernels with an fp16 w2 GEMM: the streaming kernel up to kStreamMaxT tokens
+    // (with the 64-row tiled kernel for its w2 GEMM), the tiled kernels above
+    for (int64_t T : {int64_t{1}, kStreamW2MaxT + 1, kStreamMaxT, kStreamMaxT + 1})
+        if (!make_plan(T, H, I, E, top_k, 0).act_f16) return 0;
+    // the tiled kernels address token rows with 32-bit byte offsets; the slot count is bounded as in shapes_ok
+    const int64_t by_offsets = ((int64_t{1} << 32) - 1) / (static_cast<int64_t>(H) * 2);
+    const int64_t by_slots = ((int64_t{1} << 30) - 1) / top_k;
+    const int64_t t = by_offsets < by_slots ? by_offsets : by_slots;
+    return (t > kStreamMaxT && make_plan(t, H, I, E, top_k, 0).act_f16) ? t : kStreamMaxT;
+}
+
 size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
     em_moe_layout L;
     if (em_moe_workspace_layout(T, H, I, E, top_k, flags, &L) != 0) return 0;
@@ -319,6 +342,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     // of the layer) -- but fp16 saturates at 65504 where the reference's bf16 pipeline does not, so a caller has to
     // ask for it.
     p.y_f16 = pl.y_f16 ? 1 : 0;
+    p.saturated = reinterpret_cast<int32_t*>(ws + L.saturated_off);
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
@@ -340,11 +364,12 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.sorted_len = L.sorted_len;
     p.ksplit = static_cast<int>(L.ksplit);
 
+    int32_t* counters = reinterpret_cast<int32_t*>(ws + L.tickets_off);
     const bool fused_front = !(flags & (EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN)) && norm == nullptr &&
                              gate_w == nullptr && T <= kFusedFrontMaxT && route_align_supported(T, E, top_k);
     if (fused_front) {
         rc = launch_route_align(router_logits, logits_dtype, T, top_k, renormalize, topk_w, topk_ids, p.block, sorted,
-                                L.sorted_len, eids, L.expert_ids_len, post_pad, seg_begin, s);
+                                L.sorted_len, eids, L.expert_ids_len, post_pad, seg_begin, counters, s);
         if (rc != 0) return rc;
     }
     if (!fused_front && !(flags & EM_FLAG_SKIP_ROUTER)) {
@@ -360,8 +385,12 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (rc != 0) return rc;
     }
     if (!fused_front && !(flags & EM_FLAG_SKIP_ALIGN)) {
-        rc = launch_align(topk_ids, EM_ITYPE_I32, T * top_k, E, p.block, sorted, L.sorted_len, eids,
-                          L.expert_ids_len, post_pad, seg_begin, reinterpret_cast<int32_t*>(ws + L.tickets_off), s);
+        if (T * top_k >= kMultiSortMinSlots && !(flags & EM_FLAG_ONE_GROUP_SORT))
+            rc = launch_align_multi(topk_ids, T * top_k, E, p.block, sorted, L.sorted_len, eids, L.expert_ids_len, post_pad,
+                                    seg_begin, counters, reinterpret_cast<int32_t*>(ws + L.sort_scratch_off), s);
+        else
+            rc = launch_align(topk_ids, EM_ITYPE_I32, T * top_k, E, p.block, sorted, L.sorted_len, eids,
+                              L.expert_ids_len, post_pad, seg_begin, counters, s);
         if (rc != 0) return rc;
     }
     const bool use_stream = pl.use_stream, use_tile = pl.use_tile;
@@ -370,7 +399,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
         if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
         int* tickets = (flags & EM_FLAG_NO_PERSIST) ? nullptr : reinterpret_cast<int*>(ws + L.tickets_off) + (mode - 1) * 8;
         // the sort kernel clears both launches' counters; a call that skips it (stage timing) clears them here
-        return launch_gemm_tile(q, seg_begin, mode, tickets, fused_front || (flags & EM_FLAG_SKIP_ALIGN) != 0, s);
+        return launch_gemm_tile(q, seg_begin, mode, tickets, (flags & EM_FLAG_SKIP_ALIGN) != 0, s);
     };
     if (!(flags & EM_FLAG_SKIP_GEMM1)) {
         rc = use_stream ? launch_gemm_stream(p, seg_begin, 1, s)

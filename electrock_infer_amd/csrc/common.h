@@ -11,6 +11,10 @@ namespace em {
 constexpr int kWave = 64;          // CDNA wavefront width
 constexpr int kMaxExperts = 64;    // one lane per expert in the router / sort
 constexpr int kMaxTopK = 8;
+// Counters of one layer call, one int32 each, cleared by the sort in front of the GEMMs: [0, 8) tile tickets of the
+// w13 launch, [8, 16) of the w2 launch (one per XCD), [16] activations clamped to the fp16 range.
+constexpr int kLayerCounters = 17;
+constexpr int kSaturatedCounter = 16;
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
@@ -68,6 +72,30 @@ __device__ __forceinline__ f16x8_t bf16x8_to_f16x8(bf16x8_t v) {
         out[2 * i + 1] = h[1];
     }
     return out;
+}
+// Four SiLU*mul results as fp16 bits, clamped to +-65504, for the GEMM epilogues; `seen` keeps the largest magnitude
+// bit pattern that went through (a NaN's is larger than every number's), so that the caller can tell afterwards, with
+// one compare, whether anything was clamped or was a NaN -- a NaN comes out of the clamp as a number and has to be put
+// back by the caller.  v_med3 + a packed conversion: a third of the instructions of a compare-and-select clamp.
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+constexpr uint32_t kF16MaxAsF32Bits = 0x477fe000u;  // 65504.0f
+__device__ __forceinline__ void clamp_to_f16x4(const float (&v)[4], uint32_t& seen, uint16_t (&out)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t mag = __float_as_uint(v[i]) & 0x7fffffffu;
+        seen = mag > seen ? mag : seen;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i += 2) {
+        const f32x2_t c = {__builtin_amdgcn_fmed3f(v[i], -65504.0f, 65504.0f),
+                           __builtin_amdgcn_fmed3f(v[i + 1], -65504.0f, 65504.0f)};
+        const f16x2_t h = __builtin_convertvector(c, f16x2_t);  // round to nearest even
+        uint32_t w;
+        __builtin_memcpy(&w, &h, 4);
+        out[i] = static_cast<uint16_t>(w);
+        out[i + 1] = static_cast<uint16_t>(w >> 16);
+    }
 }
 // two floats as packed fp16 (round to nearest even; clamped to the fp16 range)
 __device__ __forceinline__ uint32_t pack_f16_sat(float lo, float hi) {
@@ -144,13 +172,18 @@ int launch_norm_gate_router(const void* x_in, const void* res_in, const void* no
 int launch_align(const void* ids, int itype, int64_t numel, int E, int block,
                  int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
                  int32_t* post_pad, int32_t* seg_out /* [E+1] padded segment starts, may be null */,
-                 int32_t* tickets /* 16 tile counters to clear for the GEMM launches that follow, may be null */,
+                 int32_t* counters /* the kLayerCounters counters of a layer call to clear, may be null */,
                  hipStream_t s);
+// The same sort on several workgroups (two launches); needs align_scratch_ints(numel, E) int32 of scratch.
+int64_t align_scratch_ints(int64_t numel, int E);
+int launch_align_multi(const int32_t* ids, int64_t numel, int E, int block, int32_t* sorted, int64_t sorted_len,
+                       int32_t* expert_ids, int64_t eid_len, int32_t* post_pad, int32_t* seg_out, int32_t* counters,
+                       int32_t* scratch, hipStream_t s);
 // Router + sort in one launch (eight experts, k * T slots within the kernel's LDS table).
 bool route_align_supported(int64_t T, int E, int k);
 int launch_route_align(const void* logits, int logits_dtype, int64_t T, int k, int renorm, float* w, int32_t* ids,
                        int block, int32_t* sorted, int64_t sorted_len, int32_t* expert_ids, int64_t eid_len,
-                       int32_t* post_pad, int32_t* seg_out, hipStream_t s);
+                       int32_t* post_pad, int32_t* seg_out, int32_t* counters, hipStream_t s);
 int launch_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, hipStream_t s);
 int launch_moe_sum(const void* in, void* out, int64_t T, int topk, int64_t H, int dtype, hipStream_t s);
 bool rms_norm_supported(int H, int dtype, int weight_dtype);
@@ -170,6 +203,7 @@ struct MoeProblem {
     int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
     int y_f16;                // y holds fp16 values instead (256-row kernel, EM_FLAG_F16_PARTIALS)
+    int32_t* saturated;       // counter of activations clamped to the fp16 range (act_f16), cleared by the sort
     const int32_t* sorted_ids;
     const int32_t* expert_ids;
     const int32_t* post_pad;
@@ -184,6 +218,7 @@ struct MoeProblem {
 __device__ __forceinline__ void store_act(const MoeProblem& p, int64_t idx, float v) {
     if (p.act_f16) {
         p.act[idx] = f32_to_f16_bits_sat(v);
+        if (fabsf(v) > 65504.0f) atomicAdd(p.saturated, 1);  // rare; a NaN is not a clamped value
         return;
     }
     const uint16_t hi = f32_to_bf16_bits(v);

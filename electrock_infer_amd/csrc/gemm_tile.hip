@@ -68,9 +68,10 @@ constexpr int kDmaPerStage = 2 * kDmaHalf;              // first half A rows, se
 
 // STREAM: the weight rows are copied with the non-temporal hint.  Right when most experts fit one row tile
 // (every weight byte is then read by one workgroup only); wrong when several row tiles share them through L2.
-// F16 (w2 GEMM on fp16 activations): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
+// F16, w2 GEMM (on fp16 activations): the activation rows are fp16 (MoeProblem::act_f16); every weight fragment is turned
 // into fp16 once, before its first MFMA, and the fp16 MFMA of the same shape and rate runs instead.  F16 = 1 converts
 // bf16 weights, F16 = 2 takes weights that are fp16 in memory (MoeProblem::w2_f16) as they come.
+// F16, w13 GEMM: 1 = the SiLU*mul activations are stored as fp16 (clamped; MoeProblem::act_f16), 0 = as bf16.
 // PERSIST: the launch has one workgroup per CU (or fewer) and every workgroup walks tiles until none is left: its
 // first tile is the one its id names, the following ones come from a ticket counter per XCD (`tickets[8]`, zero
 // before the launch), so that tile i still runs on XCD i % 8 and tiles are handed out in the order above.  Nothing
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             }
     }
     auto mma = [](const bf16x8_t& a, const bf16x8_t& b, f32x4_t c) {
-        if (F16) {
+        if (MODE == 2 && F16) {
             f16x8_t ha, hb;  // the registers already hold fp16 bits
             __builtin_memcpy(&ha, &a, 16);
             __builtin_memcpy(&hb, &b, 16);
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         constexpr bool FULL = NMI == 4;
         constexpr int reads = decltype(reads_tag)::value;
         const int h = u & 1, k32 = u >> 1;
-        if (F16 == 1 && h == 0) convert_weights(k32);  // unit u is the first to use the fragments of this K half
+        if (MODE == 2 && F16 == 1 && h == 0) convert_weights(k32);  // unit u is the first to use the fragments of this K half
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (NMI ? (h * 4 + j < 2 * NMI) : (h * 4 + j < 2 * nmi)) {
@@ -518,20 +519,53 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         // act tile [256 rows][128 columns] bf16, row pitch 272 B
         constexpr int kPitchC = 128 * 2 + 16;
         {
+            // SiLU(gate) * up in float32, rounded once to the storage type, four rows of one column at a time
+            constexpr bool kAct16 = F16 != 0;
+            uint32_t seen = 0;  // largest magnitude bit pattern stored as fp16 (a NaN's is larger than any number's)
 #pragma unroll
             for (int f = 0; f < 8; ++f) {
                 if (f >= 2 * nmi) break;
 #pragma unroll
-                for (int gg = 0; gg < 2; ++gg)
+                for (int gg = 0; gg < 2; ++gg) {
+                    float v[4];
+                    uint16_t bits[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = silu_mul(acc[f][gg][i], acc[f][gg + 2][i]);
+                    if (kAct16) {
+                        clamp_to_f16x4(v, seen, bits);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) bits[i] = f32_to_bf16_bits(v[i]);
+                    }
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int row = wm * 128 + f * 16 + 4 * kq + i;
-                        const float g = acc[f][gg][i];
-                        const float u = acc[f][gg + 2][i];
-                        const float val = silu_mul(g, u);
-                        uint16_t bits = p.act_f16 ? f32_to_f16_bits_sat(val) : f32_to_bf16_bits(val);
-                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = bits;
+                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = bits[i];
                     }
+                }
+            }
+            if (kAct16 && seen > kF16MaxAsF32Bits) {
+                // rare: put the NaNs back (the clamp made numbers of them) and count the clamped values of rows
+                // that hold a routed slot (pad rows repeat token 0)
+                int n = 0;
+#pragma unroll
+                for (int f = 0; f < 8; ++f) {
+                    if (f >= 2 * nmi) break;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = wm * 128 + f * 16 + 4 * kq + i;
+                        const bool routed = p.sorted_ids[m0 + row] >= 0;
+#pragma unroll
+                        for (int gg = 0; gg < 2; ++gg) {
+                            const float val = silu_mul(acc[f][gg][i], acc[f][gg + 2][i]);
+                            if (val != val)
+                                *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = 0x7e00;
+                            else if (routed && fabsf(val) > 65504.0f)
+                                ++n;
+                        }
+                    }
+                }
+                if (n > 0) atomicAdd(p.saturated, n);
             }
             __syncthreads();
             uint16_t* dst = p.act;
@@ -557,35 +591,40 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         const int64_t yoff = static_cast<int64_t>(id_z) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
         float* ybase = p.y + yoff;
         uint16_t* ybase_h = reinterpret_cast<uint16_t*>(p.y) + yoff;  // the same partial results as fp16 (p.y_f16)
+        auto store_rows = [&](auto half_tag) {
+            constexpr bool kHalf = decltype(half_tag)::value;
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-            if (mi >= nmi) break;
+            for (int mi = 0; mi < 4; ++mi) {
+                if (mi >= nmi) break;
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh)
+                for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int row = hh * 16 + 4 * kq + i;
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = hh * 16 + 4 * kq + i;
 #pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                        *reinterpret_cast<float*>(ytile + row * kPitchY + (g * 16 + r16) * 4) = acc[mi * 2 + hh][g][i];
+                        for (int g = 0; g < 4; ++g)
+                            *reinterpret_cast<float*>(ytile + row * kPitchY + (g * 16 + r16) * 4) = acc[mi * 2 + hh][g][i];
+                    }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int row = it * 4 + (lane >> 4);
+                    const int slot = slots[wm * 128 + mi * 32 + row];
+                    f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane & 15) * 16);
+                    if (slot >= 0) {
+                        const int64_t at = static_cast<int64_t>(slot) * p.H + (lane & 15) * 4;
+                        if (kHalf)
+                            __builtin_nontemporal_store(u32x2_t{pack_f16_sat(val[0], val[1]), pack_f16_sat(val[2], val[3])},
+                                                        reinterpret_cast<u32x2_t*>(ybase_h + at));
+                        else
+                            __builtin_nontemporal_store(val, reinterpret_cast<f32x4_t*>(ybase + at));
+                    }
                 }
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int it = 0; it < 8; ++it) {
-                const int row = it * 4 + (lane >> 4);
-                const int slot = slots[wm * 128 + mi * 32 + row];
-                f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane & 15) * 16);
-                if (slot >= 0) {
-                    const int64_t at = static_cast<int64_t>(slot) * p.H + (lane & 15) * 4;
-                    if (p.y_f16)
-                        __builtin_nontemporal_store(u32x2_t{pack_f16_sat(val[0], val[1]), pack_f16_sat(val[2], val[3])},
-                                                    reinterpret_cast<u32x2_t*>(ybase_h + at));
-                    else
-                        __builtin_nontemporal_store(val, reinterpret_cast<f32x4_t*>(ybase + at));
-                }
+                __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_wave_barrier();
-        }
+        };
+        if (p.y_f16) store_rows(std::true_type{});
+        else store_rows(std::false_type{});
     }
     }  // next tile
 }
@@ -629,7 +668,11 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev].load(std::memory_order_acquire)) {
-        const void* kernels[16] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0, false>),
+        const void* kernels[20] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 1, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 1, false>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 1, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 1, true>),
+                                   reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 0, false>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0, false>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0, false>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 0, false>),
@@ -682,7 +725,8 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
             else go(gemm_tile_kernel<MODE, false, F16, false>);            \
         }                                                                  \
     } while (0)
-    if (mode == 1) EM_TILE_GO(1, 0);
+    if (mode == 1 && p.act_f16) EM_TILE_GO(1, 1);
+    else if (mode == 1) EM_TILE_GO(1, 0);
     else if (p.act_f16 && p.w2_f16) EM_TILE_GO(2, 2);
     else if (p.act_f16) EM_TILE_GO(2, 1);
     else EM_TILE_GO(2, 0);

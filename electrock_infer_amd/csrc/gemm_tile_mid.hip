@@ -68,9 +68,9 @@ __device__ __forceinline__ void wait_stages(int stages) {
 
 // One tile: `block` is the workgroup's index among those of its tile width, `col0` the first weight row
 // (MODE 1: first gate row) of the range that this width covers, `ntiles_n` the tiles across that range.
-// F16 (w2 GEMM only): the token rows are fp16 (MoeProblem::act_f16); the weight fragments are converted on their
+// F16, w2 GEMM: the token rows are fp16 (MoeProblem::act_f16); the weight fragments are converted on their
 // way from LDS to the MFMA (not when they are fp16 in memory, MoeProblem::w2_f16), which costs this HBM-bound kernel
-// nothing.
+// nothing.  F16, w13 GEMM: the SiLU*mul activations are stored as fp16 (clamped), else as bf16.
 template <int MODE, int MI, int NT, bool F16>
 __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __restrict__ seg_begin, int block, int col0,
                                           int ntiles_n, int kslice, uint8_t* smem) {
@@ -235,7 +235,7 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
     for (int kt = 0; kt + 1 < nk; ++kt) {
         if (work) {
             read_frags(smem + buf * kStageBytes, 1, 1);
-            if (F16) multiply_f16(0); else multiply(0);
+            if (MODE == 2 && F16) multiply_f16(0); else multiply(0);
         }
         {
             const int newer = nk - 2 - kt;  // stages queued after kt + 1: up to kt + kStages - 1, or the last one
@@ -247,12 +247,12 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
         buf = (buf + 1 == kStages) ? 0 : buf + 1;
         if (work) {
             read_frags(smem + buf * kStageBytes, 0, 0);
-            if (F16) multiply_f16(1); else multiply(1);
+            if (MODE == 2 && F16) multiply_f16(1); else multiply(1);
         }
     }
     if (work) {
         read_frags(smem + buf * kStageBytes, 1, 1);
-        if (F16) { multiply_f16(0); multiply_f16(1); } else { multiply(0); multiply(1); }
+        if (MODE == 2 && F16) { multiply_f16(0); multiply_f16(1); } else { multiply(0); multiply(1); }
     }
 
     // ---- epilogue through LDS (see the 256-row kernel).  Element i of lane (r16, kq) of a 16x16 accumulator is
@@ -262,18 +262,52 @@ __device__ __forceinline__ void tile_body(const MoeProblem& p, const int32_t* __
         constexpr int kColsC = NT / 2;  // act columns of the tile
         constexpr int kPitchC = kColsC * 2 + 16;
         {
+            // SiLU(gate) * up in float32, rounded once to the storage type, four rows of one column at a time
+            uint32_t seen = 0;  // largest magnitude bit pattern stored as fp16 (a NaN's is larger than any number's)
 #pragma unroll
             for (int f = 0; f < kRF; ++f) {
                 if (f >= nfr) break;
 #pragma unroll
-                for (int gg = 0; gg < kCF / 2; ++gg)
+                for (int gg = 0; gg < kCF / 2; ++gg) {
+                    float v[4];
+                    uint16_t bits[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = silu_mul(acc[f][gg][i], acc[f][gg + kCF / 2][i]);
+                    if (F16) {
+                        clamp_to_f16x4(v, seen, bits);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) bits[i] = f32_to_bf16_bits(v[i]);
+                    }
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int row = wm * (32 * MI) + f * 16 + 4 * kq + i;
-                        const float val = silu_mul(acc[f][gg][i], acc[f][gg + kCF / 2][i]);
-                        uint16_t bits = p.act_f16 ? f32_to_f16_bits_sat(val) : f32_to_bf16_bits(val);
-                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * (NT / 8) + gg * 16 + r16) * 2) = bits;
+                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * (NT / 8) + gg * 16 + r16) * 2) = bits[i];
                     }
+                }
+            }
+            if (F16 && seen > kF16MaxAsF32Bits) {
+                // rare: put the NaNs back (the clamp made numbers of them) and count the clamped values of rows
+                // that hold a routed slot (pad rows repeat token 0)
+                int n = 0;
+#pragma unroll
+                for (int f = 0; f < kRF; ++f) {
+                    if (f >= nfr) break;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = wm * (32 * MI) + f * 16 + 4 * kq + i;
+                        const bool routed = p.sorted_ids[m0 + row] >= 0;
+#pragma unroll
+                        for (int gg = 0; gg < kCF / 2; ++gg) {
+                            const float val = silu_mul(acc[f][gg][i], acc[f][gg + kCF / 2][i]);
+                            if (val != val)
+                                *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * (NT / 8) + gg * 16 + r16) * 2) = 0x7e00;
+                            else if (routed && fabsf(val) > 65504.0f)
+                                ++n;
+                        }
+                    }
+                }
+                if (n > 0) atomicAdd(p.saturated, n);
             }
             __syncthreads();
             uint16_t* dst = p.act;
@@ -383,6 +417,7 @@ bool tile_mid_supported(const MoeProblem& p) {
 // rows_per_tile: 64 or 128
 int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile, hipStream_t s) {
     if (!tile_mid_supported(p)) return EM_ERR_UNSUPPORTED;
+    if (mode == 1 && p.act_f16) return rows_per_tile == 64 ? launch_mid<1, 1, true>(p, seg_begin, s) : launch_mid<1, 2, true>(p, seg_begin, s);
     if (mode == 1) return rows_per_tile == 64 ? launch_mid<1, 1, false>(p, seg_begin, s) : launch_mid<1, 2, false>(p, seg_begin, s);
     if (p.act_f16) return rows_per_tile == 64 ? launch_mid<2, 1, true>(p, seg_begin, s) : launch_mid<2, 2, true>(p, seg_begin, s);
     return rows_per_tile == 64 ? launch_mid<2, 1, false>(p, seg_begin, s) : launch_mid<2, 2, false>(p, seg_begin, s);

@@ -186,7 +186,9 @@ class MixtralForCausalLM(nn.Module):
     @torch.no_grad()
     def init_random_weights(self, seed: int = 0, std: float = 0.02, gate_std: Optional[float] = None) -> None:
         """Explicit random initialisation (no checkpoint exists here; the reference's parameters would stay
-        torch.empty): N(0, std) for every matrix, drawn on the parameter's device expert by expert, 1 for the norms."""
+        torch.empty): N(0, std) for every matrix, drawn on the parameter's device expert by expert, 1 for the norms.
+        The draws are rounded to the model's dtype first, as a checkpoint of that dtype would hold them, and then
+        copied into the parameter (the experts' w2 may be held in another type)."""
         for li, layer in enumerate(self.model.layers):
             for name, p in layer.named_parameters():
                 g = torch.Generator(device=p.device).manual_seed(seed * 100003 + li * 101 + (zlib.crc32(name.encode()) % 97))
@@ -194,7 +196,8 @@ class MixtralForCausalLM(nn.Module):
                     p.fill_(1.0)
                 elif p.dim() == 3:
                     for e in range(p.shape[0]):
-                        p[e].copy_(torch.randn(p.shape[1:], generator=g, device=p.device, dtype=torch.float32) * std)
+                        p[e].copy_((torch.randn(p.shape[1:], generator=g, device=p.device, dtype=torch.float32) * std)
+                                   .to(self.lm_head.weight.dtype))
                 else:
                     s = gate_std if (gate_std is not None and name.endswith("gate.weight")) else std
                     p.copy_(torch.randn(p.shape, generator=g, device=p.device, dtype=torch.float32) * s)

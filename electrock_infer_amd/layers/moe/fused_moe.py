@@ -85,6 +85,11 @@ class MoeWorkspace:
     def num_tokens_post_pad(self) -> torch.Tensor:
         return self._view(self.layout.post_pad_off, 1, torch.int32)
 
+    def saturated(self) -> torch.Tensor:
+        """[1] int32: how many SiLU*mul values of routed rows the last call clamped to the fp16 range (+-65504).
+        Always 0 with ``bf16_act``; reading it (``int(ws.saturated())``) synchronises with the device."""
+        return self._view(self.layout.saturated_off, 1, torch.int32)
+
 
 # the flags the workspace size depends on
 _LAYOUT_FLAGS = _lib.FLAG_BF16_ACT | _lib.FLAG_FORCE_GENERIC

@@ -7,7 +7,12 @@ import torch
 import torch.distributed as dist
 import torch.nn as nn
 
+from ... import _lib
 from .fused_moe import fused_experts
+
+# the reference's largest batch (max_num_batched_tokens, config.py:9): w2 is kept as float16 only when every batch
+# size up to it can be served that way
+_W2_F16_MIN_TOKENS = 32768
 
 
 class FusedMoE(nn.Module):
@@ -37,15 +42,25 @@ class FusedMoE(nn.Module):
         self.renormalize = renormalize
         self.reduce_results = reduce_results
         # not in the reference: the SiLU*mul activations pass from the w13 to the w2 GEMM as fp16 (three more mantissa
-        # bits than the reference's bf16 cache2, clamped to +-65504); bf16_act=True stores them as bf16 instead
-        # (no difference in time up to 64 tokens, a few per cent faster above)
+        # bits than the reference's bf16 cache2, clamped to +-65504; a call that clamped anything says so in
+        # ``get_workspace(...).saturated()``).  bf16_act=True stores them as bf16 instead: the reference's range and
+        # rounding, the range-safe choice for checkpoints with very large activations.
         self.bf16_act = bf16_act
-        # not in the reference either: w2 kept as float16 (the loader's copy converts the bfloat16 checkpoint, exactly for
-        # every weight of magnitude 2^-14 .. 65504), which saves the w2 GEMM the conversion of its weight fragments
         if w2_dtype not in (None, torch.bfloat16, torch.float16):
             raise ValueError("w2_dtype must be bfloat16 or float16")
-        self.w2_dtype = w2_dtype
         self.params_dtype = params_dtype or torch.get_default_dtype()
+        if w2_dtype is None:
+            # not in the reference either: with bfloat16 parameters w2 is held as float16 (the loader's copy converts
+            # the checkpoint, exactly for every weight of magnitude 2^-14 .. 65504), so that the w2 GEMM multiplies
+            # the fp16 activations without converting its weight fragments (8192 tokens: -10 % on that kernel).
+            # w2_dtype=torch.bfloat16 keeps the checkpoint's type; so do bf16_act and shapes that only the
+            # shape-generic kernels take.
+            w2_dtype = self.params_dtype
+            if self.params_dtype == torch.bfloat16 and not bf16_act and intermediate_size % self.tp_size == 0 and \
+                    _lib.load().em_moe_w2_f16_max_tokens(hidden_size, intermediate_size // self.tp_size, num_experts,
+                                                         top_k) >= _W2_F16_MIN_TOKENS:
+                w2_dtype = torch.float16
+        self.w2_dtype = w2_dtype
         if self.intermediate_size % self.tp_size != 0:
             raise ValueError(f"intermediate_size ({self.intermediate_size}) must be divisible by "
                              f"tp_size ({self.tp_size})")
@@ -56,7 +71,7 @@ class FusedMoE(nn.Module):
                                        requires_grad=False)
         self.w2_weight = nn.Parameter(torch.empty(self.num_experts, self.hidden_size,
                                                   self.intermediate_size_per_partition,
-                                                  dtype=self.w2_dtype or self.params_dtype), requires_grad=False)
+                                                  dtype=self.w2_dtype), requires_grad=False)
         self.w13_weight.weight_loader = self.weight_loader
         self.w2_weight.weight_loader = self.weight_loader
 

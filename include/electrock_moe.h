@@ -52,14 +52,7 @@ extern "C" {
                                           /* as the reference stores them (default: kept finer, see below) */
 #define EM_FLAG_F16_PARTIALS   (1u << 6)  /* large batches: w2 partial sums stored as fp16 */
                                           /* (default: float32 at every batch size)                       */
-#define EM_FLAG_SKIP_ROUTER    (1u << 8)  /* stage masks: reuse what an earlier call      */
-#define EM_FLAG_SKIP_ALIGN     (1u << 9)  /* with the same shapes left in `workspace`     */
-#define EM_FLAG_SKIP_GEMM1     (1u << 10) /* (used to time one stage in isolation)        */
-#define EM_FLAG_SKIP_GEMM2     (1u << 11)
-#define EM_FLAG_SKIP_COMBINE   (1u << 12)
-#define EM_FLAG_FORCE_GENERIC  (1u << 16) /* use the shape-generic GEMM kernels           */
-#define EM_FLAG_NO_PERSIST     (1u << 17) /* diagnostic: the 256-row kernels run one workgroup per tile  */
-                                          /* instead of one per CU walking a tile queue                  */
+/* (bits 8 .. 17 are the diagnostic switches of electrock_moe_diag.h: stage masks and kernel choice) */
 
 /* Library version, e.g. 100 = 0.1.0. */
 int em_version(void);
@@ -210,9 +203,17 @@ int em_add_rms_norm(const void* x_in, const void* residual_in, void* x_out, void
                     int semantics, void* stream);
 
 /*
+ * Largest batch size T up to which every call of em_moe_forward with these weight shapes accepts
+ * EM_FLAG_W2_F16 (0: none).  The fp16 form of w2 exists in the tuned kernels only, so a caller that wants to
+ * keep w2 as fp16 (a loader deciding the storage type once, before it knows any batch size) asks here first.
+ * No counterpart in the reference, which keeps w2 in params_dtype (mixtral_moe.py:75-79).
+ */
+int64_t em_moe_w2_f16_max_tokens(int H, int I, int E, int top_k);
+
+/*
  * Bytes of device workspace em_moe_forward needs for these shapes and flags
  * (0 for invalid shapes).  The workspace must be 256-byte aligned.  The size depends on
- * EM_FLAG_BF16_ACT and EM_FLAG_FORCE_GENERIC only; pass the flags of the call.
+ * EM_FLAG_BF16_ACT (and the kernel-choice switch of electrock_moe_diag.h) only; pass the flags of the call.
  * A larger buffer than asked for is always valid: a caller that serves many batch sizes can
  * keep one workspace sized for its largest.
  */
@@ -254,7 +255,11 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigne
  * rounding of relative size 2^-12 per partial sum, mean relative error of a float32
  * output 2.1e-4 -> 3e-4).  Ignored for smaller batches.
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
- * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout).
+ * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout), and `saturated`: the number of
+ * SiLU*mul values of routed rows whose magnitude exceeded 65504 and was clamped when they were
+ * stored as fp16 (always 0 with EM_FLAG_BF16_ACT and for shapes only the generic kernels take).
+ * A caller of the default arithmetic that cannot rule such activations out reads it after the
+ * call and repeats the call with EM_FLAG_BF16_ACT when it is not 0.
  * Limits: E <= 64, top_k <= 8, H % 8 == 0, I % 8 == 0.  Unknown flag bits: EM_ERR_UNSUPPORTED.
  */
 int em_moe_forward(const void* x, const void* router_logits, int logits_dtype,
@@ -311,6 +316,8 @@ typedef struct em_moe_layout {
     int64_t post_pad_off;                          /* [1] i32                  */
     int64_t seg_begin_off;                         /* [E+1] i32 padded segment starts */
     int64_t tickets_off;                           /* [2][8] i32 tile counters of the large-batch GEMM launches */
+    int64_t saturated_off;                         /* [1] i32: activations of routed rows that the call clamped to the fp16 range */
+    int64_t sort_scratch_off;                      /* i32 histogram rows of the sort on several workgroups */
     int64_t act_off;                               /* [sorted_len, I] fp16 (bf16 with EM_FLAG_BF16_ACT and in the generic kernels) */
     int64_t act_lo_off;                            /* [sorted_len, I] bf16 rounding residuals of the generic kernels; -1: not reserved */
     int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 (fp16 with EM_FLAG_F16_PARTIALS) */

@@ -96,6 +96,12 @@ int run_case(int64_t T, int H, int I, int E, int k) {
     HIP_OK(hipMemcpy(out.data(), dout, out.size() * 4, hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(ids.data(), static_cast<char*>(dws) + L.topk_ids_off, ids.size() * 4, hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(&post_pad, static_cast<char*>(dws) + L.post_pad_off, 4, hipMemcpyDeviceToHost));
+    int32_t saturated = -1;  // activations clamped to the fp16 range: none with these operands
+    HIP_OK(hipMemcpy(&saturated, static_cast<char*>(dws) + L.saturated_off, 4, hipMemcpyDeviceToHost));
+    if (saturated != 0) {
+        std::printf("saturated counter reads %d, expected 0\n", saturated);
+        return 1;
+    }
 
     // ---- the layer on the host, in float ----
     std::vector<float> ref(T * H, 0.0f), act(I);

@@ -32,6 +32,37 @@ def test_library_exports_every_declared_symbol():
     assert b"workspace" in lib.em_error_string(-5)
 
 
+def test_diagnostic_switches_live_in_their_own_header():
+    """Stage masks and kernel-choice switches are for benchmarks and tests: the product header names none of them,
+    the binding's values are those of the diagnostic header, and no two flags share a bit."""
+    diag = open(os.path.join(ROOT, "include", "electrock_moe_diag.h")).read()
+    main = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    flags = {}
+    for text in (main, diag):
+        for name, bit in re.findall(r"#define\s+EM_FLAG_(\w+)\s+\(1u << (\d+)\)", text):
+            assert name not in flags
+            flags[name] = 1 << int(bit)
+    assert len(set(flags.values())) == len(flags)
+    for name in ("SKIP_ROUTER", "SKIP_ALIGN", "SKIP_GEMM1", "SKIP_GEMM2", "SKIP_COMBINE", "FORCE_GENERIC", "NO_PERSIST",
+                 "ONE_GROUP_SORT"):
+        assert f"EM_FLAG_{name}" not in main and f"EM_FLAG_{name}" in diag
+    for name, value in flags.items():
+        assert getattr(_lib, f"FLAG_{name}") == value, name
+
+
+def test_float16_w2_query():
+    """Which shapes may keep w2 as float16 at every batch size: those the tuned kernels take."""
+    lib = _lib.load()
+    assert lib.em_moe_w2_f16_max_tokens(4096, 14336, 8, 2) >= 32768
+    assert lib.em_moe_w2_f16_max_tokens(6144, 16384, 8, 2) >= 32768
+    assert lib.em_moe_w2_f16_max_tokens(256, 512, 8, 2) >= 32768
+    assert lib.em_moe_w2_f16_max_tokens(136, 200, 8, 2) == 0        # only the shape-generic kernels take it
+    assert lib.em_moe_w2_f16_max_tokens(4097, 512, 8, 2) == 0       # not a valid shape at all
+    # every batch size below the answer really is accepted with the flag: the layout call applies the same plan
+    for T in (1, 9, 64, 65, 32768):
+        assert lib.em_moe_workspace_bytes(T, 4096, 14336, 8, 2, _lib.FLAG_W2_F16) > 0
+
+
 def test_signatures_carry_no_torch_types():
     code = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)   # comments cite reference files
     assert "torch" not in code and "at::" not in code and "#include <hip" not in code
@@ -67,7 +98,11 @@ def test_workspace_layout_is_consistent():
         assert L.sorted_len % L.block_size == 0 and L.sorted_len >= T * 2 + 8 * (L.block_size - 1)
         assert L.expert_ids_len * L.block_size == L.sorted_len
         offs = [L.topk_weights_off, L.topk_ids_off, L.sorted_ids_off, L.expert_ids_off, L.post_pad_off,
-                L.act_off, L.y_off, L.total_bytes]
+                L.seg_begin_off, L.tickets_off, L.saturated_off, L.sort_scratch_off, L.act_off, L.y_off, L.total_bytes]
+        assert L.saturated_off == L.tickets_off + 64 and L.saturated_off % 4 == 0
+        # one histogram row per 256 ids and one per 1024, of one int32 per expert
+        assert L.act_off - L.sort_scratch_off >= -(-T * 2 // 1024) * 5 * 8 * 4
+        offs.remove(L.saturated_off)
         assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
         assert L.act_lo_off == -1                       # the tuned kernels keep no rounding residuals
         assert L.y_off - L.act_off >= L.sorted_len * I * 2

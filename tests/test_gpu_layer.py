@@ -217,6 +217,54 @@ def test_layer_8x7b_tuned_kernels_against_the_generic_kernels_on_every_row(mixtr
         assert float(d.mean()) <= (1e-6 if mode else 8e-4) * float(generic.abs().mean())
 
 
+def assert_offsets_fit(T, H, I, E=8, k=2, flags=0):
+    """Host-side bounds of a large case, checked before anything is launched: the tiled kernels form 32-bit byte
+    offsets from x, from an expert's weights and from a 256-row tile of the activations, and slot indices are int32;
+    the workspace the layout asks for must fit the device."""
+    L = _lib.workspace_layout(T, H, I, E, k, flags)
+    assert T * H * 2 < 2 ** 32 and 4 * I * H < 2 ** 32 and 256 * I * 2 < 2 ** 32
+    assert L.sorted_len < 2 ** 31 and T * k < 2 ** 30 and L.sorted_len * I < 2 ** 62
+    assert L.sorted_len == -(-(T * k + E * (L.block_size - 1)) // L.block_size) * L.block_size
+    free, _ = torch.cuda.mem_get_info()
+    assert L.total_bytes + T * H * 16 < free, (L.total_bytes, free)
+    return L
+
+
+def test_layer_8x7b_largest_engine_batch(mixtral_8x7b):
+    """T = 32768, the reference's max_num_batched_tokens (config.py:9), the largest batch its engine hands the layer:
+    routing bit-exact on all rows, the oracle on sampled rows, every row against the shape-generic kernels."""
+    T = 32768
+    announce(f"layer 8x7B T={T}")
+    m = mixtral_8x7b
+    assert_offsets_fit(T, 4096, 14336)
+    assert_offsets_fit(T, 4096, 14336, flags=_lib.FLAG_FORCE_GENERIC)
+    g = torch.Generator(device=DEV).manual_seed(77)
+    x = torch.randn(T, 4096, generator=g, device=DEV).to(torch.bfloat16)
+    lg = torch.randn(T, 8, generator=g, device=DEV)
+    ranks = torch.arange(1, 9, dtype=torch.float32) ** -1.2
+    lg = (lg + torch.log(ranks / ranks.sum())[torch.randperm(8, generator=torch.Generator().manual_seed(7))].to(DEV)).to(torch.bfloat16)
+    out = run_default(x, lg, m["w13"], m["w2"])
+    check_routing(get_workspace(DEV, T, 4096, 14336, 8, 2), lg.float().cpu(), T)
+    assert int(get_workspace(DEV, T, 4096, 14336, 8, 2).saturated()) == 0
+    rows = torch.randperm(T, generator=torch.Generator().manual_seed(5))[:96].tolist() + [0, T - 1]
+    st = error_stats(out[rows].cpu(), oracle_rows(x, lg, m["w13_cpu"], m["w2_cpu"], rows))
+    record(f"8x7b_T{T}", default=st)
+    assert st["max_abs"] <= TARGET_MAX_ABS and st["mean_rel"] <= TARGET_MEAN_REL, st
+    assert torch.isfinite(out).all()
+    out16 = fused_experts(x, m["w13"], m["w2"].to(torch.float16), lg, 2, out_dtype=torch.float32)   # the module's default
+    assert float((out16 - out).abs().max()) <= 1e-6 * float(out.abs().max())
+    del out16
+    generic = fused_experts(x, m["w13"], m["w2"], lg, 2, out_dtype=torch.float32, flags=_lib.FLAG_FORCE_GENERIC)
+    d = (out - generic).abs()
+    scale = float(generic.abs().max())
+    record(f"8x7b_T{T}_tuned_vs_generic", max_abs=float(d.max()), scale=scale, mean_abs=float(d.mean()))
+    assert float(d.max()) <= 1.5e-3 * scale and float(d.mean()) <= 8e-4 * float(generic.abs().mean())
+    from electrock_infer_amd.layers.moe.fused_moe import release_workspaces
+    del generic, d, out
+    release_workspaces()          # 6 GB of scratch that the rest of the file does not need
+    torch.cuda.empty_cache()
+
+
 def test_layer_8x7b_float16_w2(mixtral_8x7b):
     """w2 handed over as float16 at the full 8x7B shape (decode, mid-size and prefill kernels): the stated target
     against the oracle on sampled tokens."""
@@ -247,13 +295,27 @@ def test_layer_8x22b_shape():
         rows = list(range(T)) if T <= 64 else list(range(0, T, 64))
         ref = oracle_rows(xt, lt, w13_cpu, w2_cpu, rows)
         check_outputs(f"8x22b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_def[rows].cpu(), def_bf16[rows].cpu())
+    # every row of the largest batch against the shape-generic kernels, as for the 8x7B shape
+    T = 4096
+    announce(f"layer 8x22B T={T}: tuned vs generic kernels, all rows")
+    assert_offsets_fit(T, 6144, 16384)
+    for mode in (0, _lib.FLAG_BF16_ACT):
+        tuned = fused_experts(x, w13, w2, lg, 2, out_dtype=torch.float32, flags=mode)
+        generic = fused_experts(x, w13, w2, lg, 2, out_dtype=torch.float32, flags=mode | _lib.FLAG_FORCE_GENERIC)
+        d = (tuned - generic).abs()
+        scale = float(generic.abs().max())
+        record(f"8x22b_T{T}_tuned_vs_generic_flags{mode}", max_abs=float(d.max()), scale=scale, mean_abs=float(d.mean()))
+        assert float(d.max()) <= (1e-5 if mode else 1.5e-3) * scale, (mode, float(d.max()), scale)
+        assert float(d.mean()) <= (1e-6 if mode else 8e-4) * float(generic.abs().mean())
+    out16 = fused_experts(x, w13, w2.to(torch.float16), lg, 2, out_dtype=torch.float32)
+    assert float((out16 - tuned).abs().max()) <= TOL_MAX_ABS_F32 * scale     # (tuned holds the bf16-activation form here)
 
 
 def test_fusedmoe_module_runs_in_place_and_matches(mixtral_8x7b):
     announce("FusedMoE module, in place")
     m = mixtral_8x7b
     layer = FusedMoE(num_experts=8, top_k=2, hidden_size=4096, intermediate_size=14336, tp_size=1,
-                     params_dtype=torch.bfloat16, renormalize=True, reduce_results=True).to(DEV)
+                     params_dtype=torch.bfloat16, renormalize=True, reduce_results=True, w2_dtype=torch.bfloat16).to(DEV)
     layer.w13_weight.data = m["w13"]          # share storage instead of a second 2.8 GB copy
     layer.w2_weight.data = m["w2"]
     x = m["x"][:48].clone()
@@ -343,6 +405,34 @@ def test_layer_router_and_sort_in_one_launch(T, dtype):
     check_routing(get_workspace(DEV, T, 256, 512, 8, 2), lg.float(), T)
 
 
+@pytest.mark.parametrize("E,k", [(8, 2), (16, 4), (5, 1), (64, 8)])
+@pytest.mark.parametrize("T", [2048, 4096, 4097, 5000, 12289, 40000])
+@pytest.mark.parametrize("routing", ["normal", "two_experts"])
+def test_layer_sort_on_several_workgroups_writes_the_same_bytes(T, E, k, routing):
+    """From 8192 routed slots the layer sorts on several workgroups (two launches, histogram rows in the workspace):
+    every byte of sorted_token_ids, expert_ids, num_tokens_post_pad and the segment starts equals what the
+    one-workgroup kernel writes, pads and tails included, and the oracle's routing."""
+    if T * k < 8192:
+        pytest.skip("fewer than 8192 routed slots: the one-workgroup sort runs either way")
+    announce(f"sort on several workgroups: T={T} E={E} top-{k} {routing}")
+    H, I = 256, 128
+    x, lg, w13, w2 = O.make_inputs(T, H, I, E=E, seed=T + E, logits=routing)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    ws = get_workspace(DEV, T, H, I, E, k)
+    L = ws.layout
+    head = slice(0, L.act_off)                     # everything in front of the activations
+    ws.buffer[head].fill_(0x5A)
+    fused_experts(xd, w13d, w2d, lgd, k, out_dtype=torch.float32, flags=_lib.FLAG_ONE_GROUP_SORT)
+    one = ws.buffer[head].clone()
+    ws.buffer[head].fill_(0xA5)
+    fused_experts(xd, w13d, w2d, lgd, k, out_dtype=torch.float32)
+    check_routing(ws, lg.float(), T, E=E, k=k)
+    many = ws.buffer[head]
+    for off, n in ((L.sorted_ids_off, L.sorted_len), (L.expert_ids_off, L.expert_ids_len), (L.post_pad_off, 1),
+                   (L.seg_begin_off, E + 1), (L.topk_ids_off, T * k)):
+        assert torch.equal(one[off:off + 4 * n], many[off:off + 4 * n]), (off, n)
+
+
 @pytest.mark.parametrize("T", [1, 7, 33, 64, 200, 400, 777, 2100])
 def test_layer_with_float16_w2(T):
     """w2 handed over as float16 (converted once from bf16: exact in this range) runs the default mode's arithmetic
@@ -366,11 +456,13 @@ def test_layer_with_float16_w2(T):
         fused_experts(xd, w13d, w2h, lgd, 2, bf16_act=True)
 
 
-def test_fusedmoe_module_with_float16_w2():
-    announce("FusedMoE module, w2_dtype=float16")
+@pytest.mark.parametrize("w2_dtype", [None, torch.float16])
+def test_fusedmoe_module_with_float16_w2(w2_dtype):
+    """The module holds w2 as float16 by default (bfloat16 parameters, a shape the tuned kernels take)."""
+    announce(f"FusedMoE module, w2_dtype={w2_dtype}")
     x, lg, w13, w2 = O.make_inputs(70, MID["H"], MID["I"], seed=70)
     layer = FusedMoE(num_experts=8, top_k=2, hidden_size=MID["H"], intermediate_size=MID["I"], tp_size=1,
-                     params_dtype=torch.bfloat16, w2_dtype=torch.float16).to(DEV)
+                     params_dtype=torch.bfloat16, w2_dtype=w2_dtype).to(DEV)
     assert layer.w2_weight.dtype == torch.float16 and layer.w13_weight.dtype == torch.bfloat16
     for e in range(8):   # the reference loader's calls (utils/loader.py:36-49): the copy converts w2
         layer.weight_loader(layer.w13_weight, w13[e, :MID["I"]].to(DEV), "w1", e)
@@ -411,6 +503,40 @@ def test_default_mode_clamps_activations_at_the_fp16_range(T):
     assert float((out - ref).abs().max()) <= TOL_MAX_ABS_F32 * scale
     assert float((acc - ref_clamped).abs().max()) <= 1e-3 * scale
     assert float((ref - ref_clamped).abs().max()) > 20e-3 * scale      # the two definitions are well apart here
+
+
+@pytest.mark.parametrize("T", [5, 40, 100, 300, 600, 2100])
+def test_saturated_counter_reports_clamped_activations(T):
+    """A caller of the default mode can tell that activations were clamped: the workspace's `saturated` counter holds
+    the number of SiLU*mul values of routed rows beyond +-65504 after the call (streaming, 64- / 128-row and 256-row
+    kernels), and 0 after a call with ordinary magnitudes or with bf16 activations.  Padding rows do not count."""
+    announce(f"saturated counter, T={T}")
+    x, lg, w13, w2 = mid_inputs(T, "zipf", seed=1900 + T)
+    xb, w13b = (x.float() * 30).to(torch.bfloat16), (w13.float() * 50).to(torch.bfloat16)
+    I = MID["I"]
+    _, ids = O.topk_softmax(lg.float().numpy(), 2, True)
+    over, near = 0, 0
+    for e in range(8):
+        rows = np.nonzero((ids == e).any(axis=1))[0]
+        if rows.size == 0:
+            continue
+        h = xb[rows].double() @ w13b[e].double().t()
+        act = (h[:, :I] / (1.0 + torch.exp(-h[:, :I]))) * h[:, I:]
+        over += int((act.abs() > 65504).sum())
+        near += int(((act.abs() > 65504 * 0.999) & (act.abs() < 65504 * 1.001)).sum())   # the MFMA's sum may differ
+    assert over > 10 * T
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (xb, lg, w13b, w2))
+    ws = get_workspace(DEV, T, MID["H"], I, 8, 2)
+    fused_experts(xd, w13d, w2d, lgd, 2, out_dtype=torch.float32)
+    got = int(ws.saturated())
+    assert abs(got - over) <= near, (got, over, near)
+    # the next call clears the counter: bf16 activations never clamp, ordinary magnitudes do not reach the bound
+    fused_experts(xd, w13d, w2d, lgd, 2, out_dtype=torch.float32, bf16_act=True)
+    assert int(get_workspace(DEV, T, MID["H"], I, 8, 2, _lib.FLAG_BF16_ACT).saturated()) == 0
+    fused_experts(x.to(DEV), w13.to(DEV), w2d, lgd, 2, out_dtype=torch.float32)
+    assert int(ws.saturated()) == 0
+    fused_experts(xd, w13d, w2d.to(torch.float16), lgd, 2)          # the drop-in layer's form: fp16 w2, bf16 output
+    assert abs(int(ws.saturated()) - over) <= near
 
 
 def test_partial_sums_are_float32_unless_fp16_is_asked_for():

@@ -63,8 +63,10 @@ def _oracle_layer(t, l, x, residual, eps):
     return O.moe_layer_fp32(h, torch.from_numpy(logits), w13, w2), h, torch.from_numpy(np.asarray(res))
 
 
-@pytest.mark.parametrize("w2_dtype", [None, torch.float16])
+@pytest.mark.parametrize("w2_dtype", [None, torch.bfloat16])
 def test_checkpoint_loaded_onto_the_gpu_runs_the_layer(tmp_path, w2_dtype):
+    """w2_dtype=None: the module's default, w2 held as float16 (the loader's copy converts the bfloat16 checkpoint);
+    torch.bfloat16: the checkpoint's own type."""
     announce(f"load_model(device=cuda) -> MixtralMoE / PostAttentionMoE, w2_dtype={w2_dtype}")
     layers = 2
     t = _write_checkpoint(tmp_path, layers)
@@ -77,14 +79,14 @@ def test_checkpoint_loaded_onto_the_gpu_runs_the_layer(tmp_path, w2_dtype):
     for l, layer in enumerate(model.model.layers):
         ex = layer.block_sparse_moe.experts
         assert ex.w13_weight.is_cuda and ex.w2_weight.is_cuda
-        assert ex.w2_weight.dtype == (w2_dtype or torch.bfloat16) and ex.w13_weight.dtype == torch.bfloat16
+        assert ex.w2_weight.dtype == (w2_dtype or torch.float16) and ex.w13_weight.dtype == torch.bfloat16
         pre = f"model.layers.{l}."
         for e in (0, E - 1):
             assert torch.equal(ex.w13_weight[e, :I].cpu(), t[pre + f"block_sparse_moe.experts.{e}.w1.weight"])
             assert torch.equal(ex.w13_weight[e, I:].cpu(), t[pre + f"block_sparse_moe.experts.{e}.w3.weight"])
             # (a float16 parameter holds every bf16 weight of magnitude >= 2^-14 exactly, smaller ones to 2^-25)
             d = (ex.w2_weight[e].float().cpu() - t[pre + f"block_sparse_moe.experts.{e}.w2.weight"].float()).abs()
-            assert float(d.max()) <= (2.0 ** -25 if w2_dtype == torch.float16 else 0.0)
+            assert float(d.max()) <= (2.0 ** -25 if w2_dtype is None else 0.0)
         for T in (3, 70, 600):
             x = torch.randn(T, H, generator=g).to(torch.bfloat16)
             r = torch.randn(T, H, generator=g).to(torch.bfloat16)

@@ -33,6 +33,25 @@ def test_op_surface_matches_reference_binding():
     assert em._C is _C
 
 
+def test_fusedmoe_keeps_w2_as_float16_where_the_tuned_kernels_run():
+    """bfloat16 parameters: w2 is held as float16 (the w2 GEMM multiplies fp16 activations) unless the caller opts
+    out, asks for bf16 activations, uses another parameter type, or the shape falls to the shape-generic kernels."""
+    kw = dict(num_experts=8, top_k=2, hidden_size=256, intermediate_size=512, tp_size=1)
+    m = FusedMoE(**kw, params_dtype=torch.bfloat16)
+    assert m.w2_weight.dtype == torch.float16 and m.w13_weight.dtype == torch.bfloat16 and m.w2_dtype == torch.float16
+    assert FusedMoE(**kw, params_dtype=torch.bfloat16, w2_dtype=torch.bfloat16).w2_weight.dtype == torch.bfloat16
+    assert FusedMoE(**kw, params_dtype=torch.bfloat16, bf16_act=True).w2_weight.dtype == torch.bfloat16
+    assert FusedMoE(**kw, params_dtype=torch.float32).w2_weight.dtype == torch.float32
+    odd = dict(kw, hidden_size=136, intermediate_size=200)
+    assert FusedMoE(**odd, params_dtype=torch.bfloat16).w2_weight.dtype == torch.bfloat16
+    # the loader's copy converts: bf16 checkpoint values are exact in fp16 at these magnitudes
+    w2 = (torch.randn(256, 512, generator=torch.Generator().manual_seed(1)) * 0.02).to(torch.bfloat16)
+    m.weight_loader(m.w2_weight, w2, "w2", 3)
+    big = w2.float().abs() >= 2.0 ** -14
+    assert torch.equal(m.w2_weight[3].float()[big], w2.float()[big])
+    assert float((m.w2_weight[3].float() - w2.float()).abs().max()) <= 2.0 ** -25
+
+
 def test_moe_config_rule():
     assert _get_moe_config(8, 8, 14336, 2) == {"BLOCK_SIZE_M": 16, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 64,
                                                "GROUP_SIZE_M": 1}
