@@ -1,5 +1,5 @@
 """End-to-end harness around the MoE layer: a Mixtral-shaped decoder-only model with a paged KV cache, a
-prefill-first scheduler with preemption, a prefix-caching block manager and a sampler -- this build's own
+prefill-first batch planner with preemption, a prefix-reusing pool of KV blocks and a sampler -- this build's own
 counterpart of the reference's engine (electrock_infer/engine/*, models/mixtral.py, layers/sampler.py), kept small.
 
 It exists to run the MoE path inside a whole generation loop (the end-to-end configuration of the benchmark) and is

@@ -23,7 +23,7 @@ class ModelRunner:
             self.model = MixtralForCausalLM(cfg, fused_moe_tail=config.fused_moe_tail)
         self.model.init_random_weights(config.seed)
         self.sampler = Sampler()
-        # one MoE workspace for the largest batch the scheduler can form: no layer call allocates afterwards
+        # one MoE workspace for the largest batch the planner can form: no layer call allocates afterwards
         reserve_workspace(self.device, config.max_num_batched_tokens, cfg.hidden_size, cfg.intermediate_size,
                           cfg.num_local_experts, cfg.num_experts_per_tok)
         self.allocate_kv_cache()

@@ -111,6 +111,10 @@ def _ensure_buffer(device, nbytes: int) -> torch.Tensor:
     idx = _device_index(device)
     buf = _buffers.get(idx)
     if buf is None or buf.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            # an allocation made now would come from the graph's private pool and then serve eager calls as well
+            raise RuntimeError("the shared MoE workspace would have to grow under graph capture: run the layer once "
+                               "eagerly at this batch size first, or call reserve_workspace for the largest batch")
         if buf is not None:
             _retired.setdefault(idx, []).append(buf)
             nbytes = max(nbytes, buf.numel() * 3 // 2)
@@ -131,14 +135,30 @@ def release_workspaces(device=None) -> None:
     for idx in ([_device_index(device)] if device is not None else list(_buffers)):
         _buffers.pop(idx, None)
         _retired.pop(idx, None)
+        for key in [k for k in _views if k[0] == idx]:
+            del _views[key]
+
+
+_views: Dict[tuple, MoeWorkspace] = {}      # (device, shape, layout flags) -> the view handed out last
 
 
 def get_workspace(device, T: int, H: int, I: int, E: int, top_k: int, flags: int = 0) -> MoeWorkspace:
     """The layout of a call of this shape in the device's shared workspace.  Calls on one device share that buffer:
     they have to be ordered on one stream (as the layers of a model are); a caller that runs layer calls on several
-    streams at once passes each its own ``MoeWorkspace`` through the ``workspace`` argument of the entry points."""
+    streams at once passes each its own ``MoeWorkspace`` through the ``workspace`` argument of the entry points.
+    The view of a shape is kept and handed out again while the buffer behind it is still the device's current one
+    (a decode step calls this 32 times with one shape)."""
+    idx = _device_index(device)
+    key = (idx, T, H, I, E, top_k, flags & _LAYOUT_FLAGS)
+    ws = _views.get(key)
+    if ws is not None and ws.buffer is _buffers.get(idx):
+        return ws
     need = _lib.workspace_layout(T, H, I, E, top_k, flags & _LAYOUT_FLAGS).total_bytes
-    return MoeWorkspace(device, T, H, I, E, top_k, flags, buffer=_ensure_buffer(device, need))
+    ws = MoeWorkspace(device, T, H, I, E, top_k, flags, buffer=_ensure_buffer(device, need))
+    if len(_views) >= 256:
+        _views.clear()
+    _views[key] = ws
+    return ws
 
 
 def _w2_flag(w2: torch.Tensor) -> int:

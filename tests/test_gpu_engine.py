@@ -65,7 +65,7 @@ def test_greedy_generation_matches_the_float32_restatement(fused_tail):
     assert st["preemptions"] >= 1, st                                     # the small cache did force one
     assert any(c >= 64 for _, _, _, c in seen), "no prefill step found its prefix in the cache"
     assert st["prefill_steps"] >= 2 and st["decode_steps"] >= max(max_tokens) - 1
-    assert len(engine.scheduler.block_manager.free_block_ids) == 13      # everything was given back
+    assert engine.planner.pool.num_free == 13      # everything was given back
 
     # one restatement pass per request over its final tokens gives the logits of every prefix
     final = {}

@@ -98,3 +98,28 @@ def test_graphs_of_two_batch_sizes_through_the_module_share_the_workspace():
             torch.cuda.synchronize()
             assert torch.equal(buf, eager), f"replay {rep}"
     del junk
+
+
+def test_shared_workspace_refuses_to_grow_under_capture():
+    """A batch size the shared workspace has not seen, first met under capture: the buffer would be allocated from
+    the graph's private pool and then serve eager calls too, so the layer raises instead and names the remedy."""
+    from electrock_infer_amd.layers.moe import fused_moe
+    announce("graph capture, workspace growth refused")
+    H, I, E = 512, 1024, 8
+    fused_moe.release_workspaces(DEV)
+    x, lg, w13, w2 = gpu_inputs(128, H, I, E, seed=9)
+    fused_moe.fused_experts(x[:8].contiguous(), w13, w2, lg[:8].contiguous(), topk=2)      # sizes the buffer for 8 tokens
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="reserve_workspace"):
+        with torch.cuda.graph(g):
+            fused_moe.fused_experts(x, w13, w2, lg, topk=2)
+    torch.cuda.synchronize()
+    fused_moe.reserve_workspace(DEV, 128, H, I, E, 2)
+    eager = fused_moe.fused_experts(x, w13, w2, lg, topk=2).clone()
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        out = fused_moe.fused_experts(x, w13, w2, lg, topk=2)
+    g2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager)

@@ -53,6 +53,34 @@ def test_static_entry_point_matches_workspace_entry_point(H, I):
             assert torch.equal(got, want)
 
 
+def test_static_entry_point_with_the_tiled_kernels_and_changing_batch_sizes():
+    """A small shape lets batches of hundreds of tokens into the fixed array: the 64- / 128-row kernels and the 256-row
+    kernels, whose tile tickets then live in that array and are cleared by the sort in front of them.  Calls of
+    changing size in a row (large after small, small after large: the array holds whatever the call before left,
+    tickets and the saturation counter included), each against em_moe_forward on a fresh workspace with every
+    bit set: equal bit for bit."""
+    lib = _lib.load()
+    H, I, E = 512, 1024, 8
+    x, lg, w13, w2 = gpu_inputs(1024, H, I, E, seed=23)
+    w2h = w2.to(torch.float16)
+    for T, flags in ((300, 0), (1024, 0), (70, _lib.FLAG_OUT_F32), (1024, _lib.FLAG_W2_F16 | _lib.FLAG_OUT_F32), (5, 0),
+                     (600, _lib.FLAG_W2_F16), (1024, _lib.FLAG_BF16_ACT)):
+        announce(f"static entry point, tiled kernels: T={T} flags={flags}")
+        xt, lt = x[:T].contiguous(), lg[:T].contiguous()
+        w2t = w2h if flags & _lib.FLAG_W2_F16 else w2
+        odt = torch.float32 if flags & _lib.FLAG_OUT_F32 else torch.bfloat16
+        need = lib.em_moe_workspace_bytes(T, H, I, E, 2, flags)
+        assert 0 < need <= _lib.STATIC_SCRATCH_BYTES
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=DEV)
+        want = torch.full((T, H), float("nan"), dtype=odt, device=DEV)
+        got = torch.full((T, H), float("nan"), dtype=odt, device=DEV)
+        assert _forward(lib, xt, lt, w13, w2t, want, flags, ws) == 0
+        assert _forward(lib, xt, lt, w13, w2t, got, flags) == 0
+        torch.cuda.synchronize()
+        assert torch.isfinite(want.float()).all()
+        assert torch.equal(got, want)
+
+
 def test_static_entry_point_refuses_what_does_not_fit():
     lib = _lib.load()
     announce("static entry point, size limit")
