@@ -19,7 +19,7 @@ FLAG_OUT_F32 = 1 << 0
 FLAG_GATE_F32_LOGITS = 1 << 2
 FLAG_W2_F16 = 1 << 3
 FLAG_BF16_ACT = 1 << 5        # SiLU*mul activations stored as bf16 between the GEMMs (the reference's storage type)
-FLAG_F16_PARTIALS = 1 << 6    # large batches: w2 partial sums stored as fp16
+FLAG_F32_PARTIALS = 1 << 7    # w2 partial sums stored as float32 at every batch size (default: fp16 + escape above 448 tokens)
 # diagnostic switches (include/electrock_moe_diag.h): benchmarks and tests only
 FLAG_SKIP_ROUTER = 1 << 8
 FLAG_SKIP_ALIGN = 1 << 9
@@ -47,7 +47,7 @@ class MoeLayout(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in (
         "block_size", "topk_weights_off", "topk_ids_off", "sorted_ids_off", "sorted_len",
         "expert_ids_off", "expert_ids_len", "post_pad_off", "seg_begin_off", "tickets_off", "saturated_off",
-        "sort_scratch_off", "act_off", "act_lo_off", "y_off", "ksplit",
+        "sort_scratch_off", "act_off", "act_lo_off", "y_off", "ksplit", "y_wide_off",
         "total_bytes")]
 
 

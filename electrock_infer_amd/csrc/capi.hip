@@ -72,7 +72,7 @@ bool shapes_ok(int64_t T, int H, int I, int E, int top_k) {
 }
 
 constexpr unsigned kKnownFlags = EM_FLAG_OUT_F32 | EM_FLAG_GATE_F32_LOGITS | EM_FLAG_W2_F16 | EM_FLAG_BF16_ACT |
-                                 EM_FLAG_F16_PARTIALS | EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN | EM_FLAG_SKIP_GEMM1 |
+                                 EM_FLAG_F32_PARTIALS | EM_FLAG_SKIP_ROUTER | EM_FLAG_SKIP_ALIGN | EM_FLAG_SKIP_GEMM1 |
                                  EM_FLAG_SKIP_GEMM2 | EM_FLAG_SKIP_COMBINE | EM_FLAG_FORCE_GENERIC | EM_FLAG_NO_PERSIST |
                                  EM_FLAG_ONE_GROUP_SORT;
 
@@ -86,7 +86,7 @@ struct Plan {
     bool w2_on_mid;             // streaming-size batch whose w2 GEMM runs on the 64-row tiled kernel
     bool act_f16;               // SiLU*mul activations stored as fp16 (tuned kernels, default)
     bool act_pair;              // ... as a bf16 pair (value, rounding residual): generic kernels, default
-    bool y_f16;                 // w2 partial sums stored as fp16 (opt-in, 256-row kernel)
+    bool y_f16;                 // w2 partial sums stored as fp16 with a float32 escape (256-row kernel)
 };
 
 Plan make_plan(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
@@ -110,7 +110,7 @@ Plan make_plan(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
     const bool bf16_act = (flags & EM_FLAG_BF16_ACT) != 0;
     pl.act_f16 = !bf16_act && (pl.use_stream || pl.use_tile);
     pl.act_pair = !bf16_act && !pl.act_f16;
-    pl.y_f16 = (flags & EM_FLAG_F16_PARTIALS) && pl.use_tile && T > kTile128W2MaxT;
+    pl.y_f16 = !(flags & EM_FLAG_F32_PARTIALS) && pl.use_tile && T > kTile128W2MaxT;
     return pl;
 }
 
@@ -140,7 +140,8 @@ int layout_from_plan(const Plan& pl, int64_t T, int H, int I, int E, int top_k, 
     // the rounding residuals exist only where the shape-generic kernels run in the default (two-term) form
     L->act_lo_off = pl.act_pair ? take(pl.sorted_len * static_cast<int64_t>(I) * 2) : -1;
     L->ksplit = pl.ksplit;
-    L->y_off = take(pl.ksplit * slots * static_cast<int64_t>(H) * 4);
+    L->y_off = take(pl.ksplit * slots * static_cast<int64_t>(H) * (pl.y_f16 ? 2 : 4));
+    L->y_wide_off = pl.y_f16 ? take(pl.ksplit * slots * static_cast<int64_t>(H) * 4) : -1;
     L->total_bytes = off;
     return 0;
 }
@@ -335,16 +336,17 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     p.act_lo = pl.act_pair ? reinterpret_cast<uint16_t*>(ws + L.act_lo_off) : nullptr;
     p.act_f16 = pl.act_f16 ? 1 : 0;
     p.w2_f16 = (flags & EM_FLAG_W2_F16) ? 1 : 0;
-    // The partial results of the w2 GEMM (one per routed slot and K slice, before the routing weight) are float32.
-    // EM_FLAG_F16_PARTIALS stores those of the 256-row kernel as fp16 (their rounding, 2^-12, is far below a bf16
+    // The partial results of the w2 GEMM (one per routed slot and K slice, before the routing weight) are float32 up
+    // to 448 tokens.  Above, the 256-row kernel stores them as fp16 (their rounding, 2^-12, is far below a bf16
     // output's, 2^-9, and of the size of the fp16 activations'): half the bytes written by the kernel's epilogues,
-    // which all fall into the same moments of a launch, and half the bytes read by the combine (T=8192: -1 to -2.5 %
-    // of the layer) -- but fp16 saturates at 65504 where the reference's bf16 pipeline does not, so a caller has to
-    // ask for it.
+    // which all fall into the same moments of a launch, and half the bytes read by the combine (T=8192: -1 % of the
+    // layer).  A value beyond the fp16 range is stored as the fp16 infinity and, as float32, in y_wide, where the
+    // combine finds it: nothing is clamped.  EM_FLAG_F32_PARTIALS keeps float32 at every size.
     p.y_f16 = pl.y_f16 ? 1 : 0;
     p.saturated = reinterpret_cast<int32_t*>(ws + L.saturated_off);
     p.y_accumulate = 0;
     p.y = reinterpret_cast<float*>(ws + L.y_off);
+    p.y_wide = pl.y_f16 ? reinterpret_cast<float*>(ws + L.y_wide_off) : nullptr;
     int32_t* sorted = reinterpret_cast<int32_t*>(ws + L.sorted_ids_off);
     int32_t* eids = reinterpret_cast<int32_t*>(ws + L.expert_ids_off);
     int32_t* post_pad = reinterpret_cast<int32_t*>(ws + L.post_pad_off);

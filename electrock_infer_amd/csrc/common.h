@@ -80,6 +80,7 @@ __device__ __forceinline__ f16x8_t bf16x8_to_f16x8(bf16x8_t v) {
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 constexpr uint32_t kF16MaxAsF32Bits = 0x477fe000u;  // 65504.0f
+constexpr uint32_t kF16InfAsF32Bits = 0x477ff000u;  // 65520.0f: from here on a float32 rounds to the fp16 infinity
 __device__ __forceinline__ void clamp_to_f16x4(const float (&v)[4], uint32_t& seen, uint16_t (&out)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -96,10 +97,6 @@ __device__ __forceinline__ void clamp_to_f16x4(const float (&v)[4], uint32_t& se
         out[i] = static_cast<uint16_t>(w);
         out[i + 1] = static_cast<uint16_t>(w >> 16);
     }
-}
-// two floats as packed fp16 (round to nearest even; clamped to the fp16 range)
-__device__ __forceinline__ uint32_t pack_f16_sat(float lo, float hi) {
-    return static_cast<uint32_t>(f32_to_f16_bits_sat(lo)) | (static_cast<uint32_t>(f32_to_f16_bits_sat(hi)) << 16);
 }
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -202,7 +199,9 @@ struct MoeProblem {
     int w2_f16;               // w2 holds fp16 values already: the fp16 w2 kernels skip their conversion
     int y_accumulate;         // generic w2 GEMM adds to y instead of overwriting it (second pass over act_lo)
     float* y;                 // [ksplit, T*top_k, H] f32, rows by flat slot
-    int y_f16;                // y holds fp16 values instead (256-row kernel, EM_FLAG_F16_PARTIALS)
+    int y_f16;                // y holds fp16 values instead (256-row kernel); a value beyond the fp16 range is the
+                              // fp16 infinity there and stands as float32 in y_wide at the same index
+    float* y_wide;            // [ksplit, T*top_k, H] f32, written only where y holds an escaped value
     int32_t* saturated;       // counter of activations clamped to the fp16 range (act_f16), cleared by the sort
     const int32_t* sorted_ids;
     const int32_t* expert_ids;

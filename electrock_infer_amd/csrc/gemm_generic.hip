@@ -216,18 +216,21 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
     }
 }
 
-// The same sum over fp16 partial results: eight columns per thread (16-byte loads).
+// The same sum over fp16 partial results: eight columns per thread (16-byte loads).  An fp16 infinity marks a value
+// that did not fit the format; it stands as float32 at the same index of `wide` (rare: looked for only when a sum over
+// the K slices is not finite).
 template <bool kOutF32, bool kStream>
-__global__ __launch_bounds__(256) void combine_f16_kernel(const uint16_t* __restrict__ y, const float* __restrict__ w,
-                                                          void* __restrict__ out, int64_t T, int H, int top_k,
-                                                          int ksplit) {
+__global__ __launch_bounds__(256) void combine_f16_kernel(const uint16_t* __restrict__ y, const float* __restrict__ wide,
+                                                          const float* __restrict__ w, void* __restrict__ out, int64_t T,
+                                                          int H, int top_k, int ksplit) {
     const int64_t t = blockIdx.x;
     const int64_t zstride = T * top_k * static_cast<int64_t>(H);
     for (int h = (blockIdx.y * 256 + threadIdx.x) * 8; h < H; h += gridDim.y * 256 * 8) {
         float acc[8] = {};
         for (int j = 0; j < top_k; ++j) {
             const float wj = w[t * top_k + j];
-            const uint16_t* row = y + (t * top_k + j) * static_cast<int64_t>(H) + h;
+            const int64_t at = (t * top_k + j) * static_cast<int64_t>(H) + h;
+            const uint16_t* row = y + at;
             float s[8] = {};
             for (int z = 0; z < ksplit; ++z) {
                 const u32x4_t* ptr = reinterpret_cast<const u32x4_t*>(row + z * zstride);
@@ -237,6 +240,22 @@ __global__ __launch_bounds__(256) void combine_f16_kernel(const uint16_t* __rest
                     s[2 * i] += f16_bits_to_f32(static_cast<uint16_t>(v[i]));
                     s[2 * i + 1] += f16_bits_to_f32(static_cast<uint16_t>(v[i] >> 16));
                 }
+            }
+            uint32_t seen = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t mag = __float_as_uint(s[i]) & 0x7fffffffu;
+                seen = mag > seen ? mag : seen;
+            }
+            if (seen >= 0x7f800000u) {  // an infinity or a NaN among the sums: add again, escaped values from `wide`
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s[i] = 0.0f;
+                for (int z = 0; z < ksplit; ++z)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const uint16_t bits = row[z * zstride + i];
+                        s[i] += ((bits & 0x7fffu) == 0x7c00u) ? wide[at + z * zstride + i] : f16_bits_to_f32(bits);
+                    }
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[i] += wj * s[i];
@@ -286,8 +305,8 @@ int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s) {
         const unsigned cols = static_cast<unsigned>(ceil_div(p.H, 2048));
         const dim3 grid(static_cast<unsigned>(p.T), cols < 8 ? cols : 8);
         auto go = [&](auto kernel) {
-            launch(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.topk_w, out, p.T, p.H,
-                   p.top_k, p.ksplit);
+            launch(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint16_t*>(p.y), p.y_wide, p.topk_w, out, p.T,
+                   p.H, p.top_k, p.ksplit);
         };
         if (out_f32) { if (stream) go(combine_f16_kernel<true, true>); else go(combine_f16_kernel<true, false>); }
         else { if (stream) go(combine_f16_kernel<false, true>); else go(combine_f16_kernel<false, false>); }

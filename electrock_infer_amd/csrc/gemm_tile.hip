@@ -214,8 +214,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     bool live[kDmaPerStage];
     const uint16_t* wbase = (MODE == 1) ? p.w13 + static_cast<int64_t>(expert) * 2 * p.I * p.H
                                         : p.w2 + static_cast<int64_t>(expert) * p.H * p.I;
-    const uint8_t* base_a = reinterpret_cast<const uint8_t*>(((MODE == 1) ? p.x : p.act + m0 * static_cast<int64_t>(p.I)) + k_begin);
-    const uint8_t* base_b = reinterpret_cast<const uint8_t*>(wbase + k_begin);
+    // (wave-uniform addresses, said so to the compiler: the copies take their base from scalar registers)
+    auto uniform_ptr = [](const void* ptr) {
+        const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+        const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+        return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+    };
+    const uint8_t* base_a = uniform_ptr(((MODE == 1) ? p.x : p.act + m0 * static_cast<int64_t>(p.I)) + k_begin);
+    const uint8_t* base_b = uniform_ptr(wbase + k_begin);
 #pragma unroll
     for (int n = 0; n < kDmaPerStage; ++n) {
         const int o = (n % kDmaHalf) * 8192 + wave * 1024 + lane * 16;
@@ -295,14 +302,20 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     const int r16 = lane & 15;
     const int kq = lane >> 4;
     const int sw = (r16 >> 1) & 7;  // (row / 2) & 7 is the same for every fragment of this lane
-    int a_off[2], b_off[2];
-#pragma unroll
-    for (int k32 = 0; k32 < 2; ++k32) {
-        const int piece = (k32 * 4 + kq) ^ sw;
+    // (K half 1 reads piece (4 + kq) ^ sw = (kq ^ sw) ^ 4: its offsets are those of K half 0 with bit 6 flipped, formed
+    // where they are used instead of being kept in two more registers)
+    int a_off0, b_off0;
+    {
+        const int piece = kq ^ sw;
         const int ra = wm * 128 + r16, rb = wn * 64 + r16;
-        a_off[k32] = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
-        b_off[k32] = kOffB + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
+        a_off0 = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
+        b_off0 = kOffB + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
     }
+    struct HalfOffset {
+        int base;
+        __device__ __forceinline__ int operator[](int k32) const { return k32 ? (base ^ 64) : base; }
+    };
+    const HalfOffset a_off{a_off0}, b_off{b_off0};
     // 32-row blocks of this wave that hold rows of the tile (wave-uniform); 16-row fragment f exists if f < 2 * nmi
     int nmi = (valid - wm * 128 + 31) / 32;
     nmi = nmi < 0 ? 0 : (nmi > 4 ? 4 : nmi);
@@ -515,6 +528,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     // column per lane.  Results are turned through LDS (free after the last stage) so that global stores
     // are 16 bytes per lane on full 128-byte lines.
     block_barrier();  // every wave has read its last operands: the stage buffers can be reused
+    // (the lane's position in the tile, worked out again from the thread index instead of being kept through the
+    // main loop, which has no register to spare)
+    int tid_epi = threadIdx.x;
+    if (PERSIST) asm volatile("" : "+v"(tid_epi));
+    const int e_tid = tid_epi, e_lane = tid_epi & 63, e_r16 = tid_epi & 15, e_kq = (tid_epi >> 4) & 3;
     if (MODE == 1) {
         // act tile [256 rows][128 columns] bf16, row pitch 272 B
         constexpr int kPitchC = 128 * 2 + 16;
@@ -539,8 +557,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     }
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = wm * 128 + f * 16 + 4 * kq + i;
-                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = bits[i];
+                        const int row = wm * 128 + f * 16 + 4 * e_kq + i;
+                        *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + e_r16) * 2) = bits[i];
                     }
                 }
             }
@@ -553,13 +571,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     if (f >= 2 * nmi) break;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = wm * 128 + f * 16 + 4 * kq + i;
+                        const int row = wm * 128 + f * 16 + 4 * e_kq + i;
                         const bool routed = p.sorted_ids[m0 + row] >= 0;
 #pragma unroll
                         for (int gg = 0; gg < 2; ++gg) {
                             const float val = silu_mul(acc[f][gg][i], acc[f][gg + 2][i]);
                             if (val != val)
-                                *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + r16) * 2) = 0x7e00;
+                                *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + e_r16) * 2) = 0x7e00;
                             else if (routed && fabsf(val) > 65504.0f)
                                 ++n;
                         }
@@ -571,7 +589,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
             uint16_t* dst = p.act;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int c = tid + i * kThreads;  // 16-byte piece c of the tile: row c/16, columns (c%16)*8..+8
+                const int c = e_tid + i * kThreads;  // 16-byte piece c of the tile: row c/16, columns (c%16)*8..+8
                 const int row = c >> 4;
                 if (row < valid)
                     // (non-temporal: the tile is not read again before the w2 GEMM; as ordinary stores the activations
@@ -586,11 +604,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         constexpr int kPitchY = 64 * 4 + 16;
         int32_t* slots = reinterpret_cast<int32_t*>(smem);
         uint8_t* ytile = smem + 1024 + wave * (32 * kPitchY);
-        if (tid < kTM) slots[tid] = my_slot;
+        if (e_tid < kTM) slots[e_tid] = my_slot;
         __syncthreads();
         const int64_t yoff = static_cast<int64_t>(id_z) * p.T * p.top_k * p.H + nt * kTN + wn * 64;
         float* ybase = p.y + yoff;
         uint16_t* ybase_h = reinterpret_cast<uint16_t*>(p.y) + yoff;  // the same partial results as fp16 (p.y_f16)
+        // kHalf: the partial sums go out as fp16.  A value beyond the fp16 range becomes the fp16 infinity (the plain
+        // rounding) and is stored again as float32 at the same index of y_wide, where the combine looks when it meets
+        // an infinity: the rows of a 32-row block whose e_lane saw such a value are walked a second time (rare).
+        float* wbase_y = p.y_wide + yoff;
         auto store_rows = [&](auto half_tag) {
             constexpr bool kHalf = decltype(half_tag)::value;
 #pragma unroll
@@ -600,24 +622,45 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                 for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = hh * 16 + 4 * kq + i;
+                        const int row = hh * 16 + 4 * e_kq + i;
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
-                            *reinterpret_cast<float*>(ytile + row * kPitchY + (g * 16 + r16) * 4) = acc[mi * 2 + hh][g][i];
+                            *reinterpret_cast<float*>(ytile + row * kPitchY + (g * 16 + e_r16) * 4) = acc[mi * 2 + hh][g][i];
                     }
                 __builtin_amdgcn_wave_barrier();
+                uint32_t seen = 0;  // largest magnitude bit pattern this e_lane stored as fp16
 #pragma unroll
                 for (int it = 0; it < 8; ++it) {
-                    const int row = it * 4 + (lane >> 4);
+                    const int row = it * 4 + (e_lane >> 4);
                     const int slot = slots[wm * 128 + mi * 32 + row];
-                    f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (lane & 15) * 16);
+                    f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (e_lane & 15) * 16);
                     if (slot >= 0) {
-                        const int64_t at = static_cast<int64_t>(slot) * p.H + (lane & 15) * 4;
-                        if (kHalf)
-                            __builtin_nontemporal_store(u32x2_t{pack_f16_sat(val[0], val[1]), pack_f16_sat(val[2], val[3])},
-                                                        reinterpret_cast<u32x2_t*>(ybase_h + at));
-                        else
+                        const int64_t at = static_cast<int64_t>(slot) * p.H + (e_lane & 15) * 4;
+                        if (kHalf) {
+                            const f16x2_t lo = __builtin_convertvector(f32x2_t{val[0], val[1]}, f16x2_t);
+                            const f16x2_t hi = __builtin_convertvector(f32x2_t{val[2], val[3]}, f16x2_t);
+                            uint32_t plo, phi;
+                            __builtin_memcpy(&plo, &lo, 4);
+                            __builtin_memcpy(&phi, &hi, 4);
+                            __builtin_nontemporal_store(u32x2_t{plo, phi}, reinterpret_cast<u32x2_t*>(ybase_h + at));
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) {
+                                const uint32_t mag = __float_as_uint(val[c]) & 0x7fffffffu;
+                                seen = mag > seen ? mag : seen;
+                            }
+                        } else {
                             __builtin_nontemporal_store(val, reinterpret_cast<f32x4_t*>(ybase + at));
+                        }
+                    }
+                }
+                if (kHalf && seen >= kF16InfAsF32Bits) {
+#pragma unroll
+                    for (int it = 0; it < 8; ++it) {
+                        const int row = it * 4 + (e_lane >> 4);
+                        const int slot = slots[wm * 128 + mi * 32 + row];
+                        const f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (e_lane & 15) * 16);
+                        if (slot >= 0)
+                            *reinterpret_cast<f32x4_t*>(wbase_y + static_cast<int64_t>(slot) * p.H + (e_lane & 15) * 4) = val;
                     }
                 }
                 __builtin_amdgcn_wave_barrier();
@@ -668,7 +711,7 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!attr_set[dev].load(std::memory_order_acquire)) {
-        const void* kernels[20] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 1, false>),
+        const void* kernels[18] = {reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 1, false>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 1, false>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<1, false, 1, true>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 1, true>),
@@ -684,8 +727,6 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
                                    reinterpret_cast<const void*>(gemm_tile_kernel<1, true, 0, true>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 0, true>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 0, true>),
-                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 1, true>),
-                                   reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 1, true>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<2, false, 2, true>),
                                    reinterpret_cast<const void*>(gemm_tile_kernel<2, true, 2, true>)};
         for (const void* k : kernels) {
@@ -703,7 +744,10 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
     const bool stream_b = p.T * p.top_k * 8 <= static_cast<int64_t>(p.E) * kTM * (mode == 1 ? 7 : 10);
     const int nz = (mode == 1) ? 1 : p.ksplit;
     const int kslice = (mode == 1) ? p.H : p.I / p.ksplit;
-    const bool persist = tickets != nullptr;
+    // (the w2 kernel that converts bf16 weight fragments on the way has no register left for the tile queue: it runs
+    // one workgroup per tile; the loader's float16 w2 and bf16 activations take the queue)
+    const bool converts = mode == 2 && p.act_f16 && !p.w2_f16;
+    const bool persist = tickets != nullptr && !converts;
     dim3 g(grid, static_cast<unsigned>(nz));
     if (persist) {
         // one workgroup per CU (a workgroup takes all of a CU's LDS), a multiple of 8 so that ids map to XCDs
@@ -728,8 +772,10 @@ int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, in
     if (mode == 1 && p.act_f16) EM_TILE_GO(1, 1);
     else if (mode == 1) EM_TILE_GO(1, 0);
     else if (p.act_f16 && p.w2_f16) EM_TILE_GO(2, 2);
-    else if (p.act_f16) EM_TILE_GO(2, 1);
-    else EM_TILE_GO(2, 0);
+    else if (p.act_f16) {
+        if (stream_b) go(gemm_tile_kernel<2, true, 1, false>);
+        else go(gemm_tile_kernel<2, false, 1, false>);
+    } else EM_TILE_GO(2, 0);
 #undef EM_TILE_GO
     return launch_status();
 }

@@ -92,7 +92,7 @@ class MoeWorkspace:
 
 
 # the flags the workspace size depends on
-_LAYOUT_FLAGS = _lib.FLAG_BF16_ACT | _lib.FLAG_FORCE_GENERIC
+_LAYOUT_FLAGS = _lib.FLAG_BF16_ACT | _lib.FLAG_FORCE_GENERIC | _lib.FLAG_F32_PARTIALS
 
 # One grow-only buffer per device.  A buffer that has been handed out is never freed behind the caller's back:
 # a HIP graph captured through the layer calls holds its address, so when a larger batch makes the buffer grow,

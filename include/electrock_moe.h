@@ -50,8 +50,8 @@ extern "C" {
 #define EM_FLAG_W2_F16         (1u << 3)  /* `w2` holds fp16 values (converted once by the caller)        */
 #define EM_FLAG_BF16_ACT       (1u << 5)  /* SiLU*mul activations rounded to bf16 between the two GEMMs,  */
                                           /* as the reference stores them (default: kept finer, see below) */
-#define EM_FLAG_F16_PARTIALS   (1u << 6)  /* large batches: w2 partial sums stored as fp16 */
-                                          /* (default: float32 at every batch size)                       */
+#define EM_FLAG_F32_PARTIALS   (1u << 7)  /* w2 partial sums stored as float32 at every batch size        */
+                                          /* (default: fp16 with a float32 escape above 448 tokens)       */
 /* (bits 8 .. 17 are the diagnostic switches of electrock_moe_diag.h: stage masks and kernel choice) */
 
 /* Library version, e.g. 100 = 0.1.0. */
@@ -213,7 +213,7 @@ int64_t em_moe_w2_f16_max_tokens(int H, int I, int E, int top_k);
 /*
  * Bytes of device workspace em_moe_forward needs for these shapes and flags
  * (0 for invalid shapes).  The workspace must be 256-byte aligned.  The size depends on
- * EM_FLAG_BF16_ACT (and the kernel-choice switch of electrock_moe_diag.h) only; pass the flags of the call.
+ * EM_FLAG_BF16_ACT, EM_FLAG_F32_PARTIALS (and the kernel-choice switch of electrock_moe_diag.h) only; pass the flags of the call.
  * A larger buffer than asked for is always valid: a caller that serves many batch sizes can
  * keep one workspace sized for its largest.
  */
@@ -249,11 +249,14 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigne
  * are loaded).  Same results as the default without the conversion: within 1-2 % of
  * EM_FLAG_BF16_ACT's time at every batch size.  Only shapes the tuned kernels take and not
  * together with EM_FLAG_BF16_ACT; others return EM_ERR_UNSUPPORTED.
- * EM_FLAG_F16_PARTIALS: above 448 tokens the partial sums of the w2 GEMM (one per routed
- * slot and K slice, before the routing weight) are stored as fp16 and saturate at +-65504,
- * where the reference's bf16 pipeline does not (T=8192: -2 to -5 % in time; one more
- * rounding of relative size 2^-12 per partial sum, mean relative error of a float32
- * output 2.1e-4 -> 3e-4).  Ignored for smaller batches.
+ * Partial sums of the w2 GEMM (one per routed slot and K slice, before the routing weight): float32 up to 448
+ * tokens; above, the 256-row kernel stores them as fp16 (half the bytes in its epilogues and in the top-k sum;
+ * one more rounding of relative size 2^-12 per partial sum: mean relative error of a float32 output 2.1e-4 -> 2.9e-4).
+ * No value is clamped: a partial sum beyond the fp16 range (and an infinity) is marked by the fp16 infinity and
+ * kept as float32 in a second array of the workspace, from where the top-k sum takes it, so the layer follows the
+ * definition at any magnitude bf16 holds.  What fp16 cannot keep is relative precision below 2^-14: partial sums
+ * smaller than that in magnitude carry an absolute error of up to 2^-25.
+ * EM_FLAG_F32_PARTIALS stores float32 partial sums at every batch size (8192 tokens: +1 % in time).
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout), and `saturated`: the number of
  * SiLU*mul values of routed rows whose magnitude exceeded 65504 and was clamped when they were
@@ -320,7 +323,8 @@ typedef struct em_moe_layout {
     int64_t sort_scratch_off;                      /* i32 histogram rows of the sort on several workgroups */
     int64_t act_off;                               /* [sorted_len, I] fp16 (bf16 with EM_FLAG_BF16_ACT and in the generic kernels) */
     int64_t act_lo_off;                            /* [sorted_len, I] bf16 rounding residuals of the generic kernels; -1: not reserved */
-    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32 (fp16 with EM_FLAG_F16_PARTIALS) */
+    int64_t y_off, ksplit;                         /* [ksplit, T*top_k, H] f32, or fp16 (large batches without EM_FLAG_F32_PARTIALS) */
+    int64_t y_wide_off;                            /* [ksplit, T*top_k, H] f32 holding the partial sums that fp16 marks as escaped; -1: y is f32 */
     int64_t total_bytes;
 } em_moe_layout;
 

@@ -35,7 +35,7 @@ def test_rows_of_the_printed_line_stay_short():
     the roofline, its nested prefill object and the CPU baseline) and 25 rows, which must fit with room to spare."""
     sys.path.insert(0, ROOT)
     import bench
-    r = {"shape": "8x22b", "T": 8192, "logits": "two_experts", "mode": "bf16_act_f16_partials", "ms": 4.8123456789,
+    r = {"shape": "8x22b", "T": 8192, "logits": "two_experts", "mode": "f32_partials_f32out", "ms": 4.8123456789,
          "tokens_per_s": 1702345.678, "hbm_frac": 0.07712345, "mfma_frac": 0.4812345,
          "errors": {"max_abs": 0.00329732894, "mean_rel": 0.000213456789}, "meets_tolerance": False}
     row = json.dumps(bench.compact(r), separators=(",", ":"))
