@@ -447,14 +447,15 @@ def main():
 
     detail = []
     if not args.no_table:
-        half_steps, half_warm = max(20, args.steps // 2), max(5, args.warmup // 2)
+        # (the rows' own step counts: short runs of a few calls right after a change of batch size scatter by 10 %)
+        half_steps, half_warm = max(50, args.steps // 2), max(10, args.warmup // 2)
         big = 8192 if args.shape == "8x7b" else 4096
         # the tolerance-meeting mode at every named batch size
         for t in ((1, 8, 32, 64, 256, 512, 1024, 2048) if args.shape == "8x7b" else (1, 64)):
             if t != T or args.mode != "default_f32out":
-                detail.append(measure(torch, t, weights, half_steps if t <= 256 else 20, half_warm, host=err_host))
+                detail.append(measure(torch, t, weights, half_steps if t <= 256 else 30, half_warm, host=err_host))
         for lgk in (("normal", "zipf", "two_experts") if args.shape == "8x7b" else ("normal",)):
-            detail.append(measure(torch, big, weights, 10, 3, logits=lgk, host=err_host, stages=lgk == "normal"))
+            detail.append(measure(torch, big, weights, 20, 5, logits=lgk, host=err_host, stages=lgk == "normal"))
             if lgk == "normal":
                 pre = w13_roofline(detail[-1])
                 g2_ms = detail[-1]["stage_ms"]["gemm2"]
@@ -468,7 +469,7 @@ def main():
             if mode != args.mode:
                 detail.append(measure(torch, T, weights, half_steps, half_warm, mode=mode, host=err_host))
         for mode in ("default", "w2_bf16_f32out", "f32_partials_f32out", "bf16_act"):
-            detail.append(measure(torch, big, weights, 10, 3, mode=mode, host=err_host))
+            detail.append(measure(torch, big, weights, 20, 5, mode=mode, host=err_host))
 
     cpu = None if (args.no_cpu or host is None) else cpu_baseline(torch, T, dev, host)
     rows = [compact(r) for r in detail]
@@ -481,7 +482,7 @@ def main():
         w22 = Weights(*make_weights(torch, dev, seed=22))
         host22 = None if args.no_errors else HostWeights(w22)
         for t in (1, 64, 4096):
-            detail.append(measure(torch, t, w22, 20 if t <= 64 else 10, 5 if t <= 64 else 3, host=host22))
+            detail.append(measure(torch, t, w22, 50 if t <= 64 else 20, 10 if t <= 64 else 5, host=host22))
             rows.append(compact(detail[-1]))
         del w22, host22
         set_shape(args.shape)
