@@ -246,9 +246,11 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigne
  * 1.7e-3; no conversions in the w2 GEMM (8192 tokens: -10 % on that kernel, no difference
  * up to 64 tokens).
  * EM_FLAG_W2_F16: the caller keeps w2 as fp16 (converted once, e.g. when the weights
- * are loaded).  Same results as the default without the conversion: within 1-2 % of
- * EM_FLAG_BF16_ACT's time at every batch size.  Only shapes the tuned kernels take and not
- * together with EM_FLAG_BF16_ACT; others return EM_ERR_UNSUPPORTED.
+ * are loaded; what the FusedMoE module of this package does for bfloat16 parameters).  Same
+ * results as flags = 0 without the conversion (8192 tokens: -2.3 % of the layer) and with the tile
+ * queue in the w2 launch, which the converting kernel has no register left for.  Only shapes the
+ * tuned kernels take (em_moe_w2_f16_max_tokens) and not together with EM_FLAG_BF16_ACT; others
+ * return EM_ERR_UNSUPPORTED.
  * Partial sums of the w2 GEMM (one per routed slot and K slice, before the routing weight): float32 up to 448
  * tokens; above, the 256-row kernel stores them as fp16 (half the bytes in its epilogues and in the top-k sum;
  * one more rounding of relative size 2^-12 per partial sum: mean relative error of a float32 output 2.1e-4 -> 2.9e-4).
@@ -256,7 +258,7 @@ size_t em_moe_workspace_bytes(int64_t T, int H, int I, int E, int top_k, unsigne
  * kept as float32 in a second array of the workspace, from where the top-k sum takes it, so the layer follows the
  * definition at any magnitude bf16 holds.  What fp16 cannot keep is relative precision below 2^-14: partial sums
  * smaller than that in magnitude carry an absolute error of up to 2^-25.
- * EM_FLAG_F32_PARTIALS stores float32 partial sums at every batch size (8192 tokens: +1 % in time).
+ * EM_FLAG_F32_PARTIALS stores float32 partial sums at every batch size (8192 tokens: +1.4 % in time).
  * After the call the workspace holds topk_weights, topk_ids, sorted_token_ids,
  * expert_ids and num_tokens_post_pad (see em_moe_workspace_layout), and `saturated`: the number of
  * SiLU*mul values of routed rows whose magnitude exceeded 65504 and was clamped when they were
