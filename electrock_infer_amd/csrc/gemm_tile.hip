@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     int a_off0, b_off0;
     {
         const int piece = kq ^ sw;
-        const int ra = wm * 128 + r16, rb = wn * 64 + r16;
+        const int ra = wm * 32 + r16, rb = wn * 64 + r16;
         a_off0 = (ra >> 1) * 256 + ((ra & 1) * 8 + piece) * 16;
         b_off0 = kOffB + (rb >> 1) * 256 + ((rb & 1) * 8 + piece) * 16;
     }
@@ -316,10 +316,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         __device__ __forceinline__ int operator[](int k32) const { return k32 ? (base ^ 64) : base; }
     };
     const HalfOffset a_off{a_off0}, b_off{b_off0};
-    // 32-row blocks of this wave that hold rows of the tile (wave-uniform); 16-row fragment f exists if f < 2 * nmi
-    int nmi = (valid - wm * 128 + 31) / 32;
-    nmi = nmi < 0 ? 0 : (nmi > 4 ? 4 : nmi);
+    // The 32-row blocks of a tile are dealt alternately to the two wave rows: block b belongs to wave row b % 2, so a
+    // tile of nb blocks gives them ceil(nb / 2) and floor(nb / 2) -- with the upper and lower half of the tile instead, a
+    // tile of 128 rows kept four of the eight waves busy for as long as a full one.  16-row fragment f of wave row wm
+    // (f < 2 * nmi, nmi = the wave's blocks, wave-uniform) starts at tile row frag_row(f).
+    const int nblocks = valid / kRowBlock;
+    int nmi = (wm == 0) ? (nblocks + 1) / 2 : nblocks / 2;
     nmi = __builtin_amdgcn_readfirstlane(nmi);
+    auto frag_row = [&](int f) { return (f >> 1) * 64 + wm * 32 + (f & 1) * 16; };
+    auto frag_off = [](int f) { return (f >> 1) * 8192 + (f & 1) * 2048; };  // bytes in a slot of token rows, from fragment 0
 
     // Unit u = 0..3 of a K step: row half h = u & 1 (fragments 4h .. 4h+3), K half k32 = u >> 1.
     // Token fragments live in register set u & 1, weight fragments (shared by both row halves) in set k32.
@@ -361,7 +366,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (NMI ? (h * 4 + j < 2 * NMI) : (h * 4 + j < 2 * nmi))
-                fa[h][j] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[k32] + (h * 4 + j) * 2048);
+                fa[h][j] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[k32] + frag_off(h * 4 + j));
         if (h == 0) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) fb[k32][g] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[k32] + g * 2048);
@@ -464,7 +469,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                 } else if (n < 5) {
                     fb[0][n - 1] = *reinterpret_cast<const bf16x8_t*>(sb + b_off[0] + (n - 1) * 2048);
                 } else if (n - 4 < 2 * NMI) {
-                    fa[0][n - 4] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0] + (n - 4) * 2048);
+                    fa[0][n - 4] = *reinterpret_cast<const bf16x8_t*>(sa + a_off[0] + frag_off(n - 4));
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -494,7 +499,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     } else if (nmi == 1) {
         main_loop(std::integral_constant<int, 1>{});
     } else {
-        // A wave without rows (the tile is at most 128 rows high) still copies and meets the barriers.
+        // A wave without rows (the tile is one block high) still copies and meets the barriers.
         // Skipped copies of missing token rows do not change the counts: the newest four are B's.
         const std::integral_constant<int, 0> part;
         const bool work = nmi > 0;
@@ -557,7 +562,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     }
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = wm * 128 + f * 16 + 4 * e_kq + i;
+                        const int row = frag_row(f) + 4 * e_kq + i;
                         *reinterpret_cast<uint16_t*>(smem + row * kPitchC + (wn * 32 + gg * 16 + e_r16) * 2) = bits[i];
                     }
                 }
@@ -571,7 +576,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
                     if (f >= 2 * nmi) break;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = wm * 128 + f * 16 + 4 * e_kq + i;
+                        const int row = frag_row(f) + 4 * e_kq + i;
                         const bool routed = p.sorted_ids[m0 + row] >= 0;
 #pragma unroll
                         for (int gg = 0; gg < 2; ++gg) {
@@ -632,7 +637,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
 #pragma unroll
                 for (int it = 0; it < 8; ++it) {
                     const int row = it * 4 + (e_lane >> 4);
-                    const int slot = slots[wm * 128 + mi * 32 + row];
+                    const int slot = slots[(2 * mi + wm) * 32 + row];
                     f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (e_lane & 15) * 16);
                     if (slot >= 0) {
                         const int64_t at = static_cast<int64_t>(slot) * p.H + (e_lane & 15) * 4;
@@ -657,7 +662,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
 #pragma unroll
                     for (int it = 0; it < 8; ++it) {
                         const int row = it * 4 + (e_lane >> 4);
-                        const int slot = slots[wm * 128 + mi * 32 + row];
+                        const int slot = slots[(2 * mi + wm) * 32 + row];
                         const f32x4_t val = *reinterpret_cast<const f32x4_t*>(ytile + row * kPitchY + (e_lane & 15) * 16);
                         if (slot >= 0)
                             *reinterpret_cast<f32x4_t*>(wbase_y + static_cast<int64_t>(slot) * p.H + (e_lane & 15) * 4) = val;
