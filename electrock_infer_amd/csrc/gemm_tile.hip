@@ -31,7 +31,7 @@
 //              limit, not the issue rate, sets the speed, and this shape needs less power
 //              per flop (registers-only loop, N(0,1) x N(0,0.02) operands: 2.08 against
 //              1.85 PFLOP/s for 32x32x16).  A K step of 64 is walked in four units of 16
-//              MFMAs (upper / lower 64 rows x first / second 32 of K); operand fragments are
+//              MFMAs (first / second two 32-row blocks of the wave x first / second 32 of K); operand fragments are
 //              double-buffered in registers and their LDS reads are woven between the
 //              MFMAs of the previous unit, also across the stage barrier
 //   MODE 1     N fragments 0, 1 of a wave are 32 gate rows j and fragments 2, 3 the matching
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
         for (int n = 0; n < kDmaHalf; ++n) copy_b(n, stage_k, slot);
     };
 
-    // accumulator (f, g): rows wm*128 + f*16 .. +16 of the tile, weight rows wn*64 + g*16 .. +16
+    // accumulator (f, g): rows frag_row(f) .. +16 of the tile (see below), weight rows wn*64 + g*16 .. +16
     f32x4_t acc[8][4];
 #pragma unroll
     for (int f = 0; f < 8; ++f)
@@ -317,8 +317,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(MoeProblem p, co
     };
     const HalfOffset a_off{a_off0}, b_off{b_off0};
     // The 32-row blocks of a tile are dealt alternately to the two wave rows: block b belongs to wave row b % 2, so a
-    // tile of nb blocks gives them ceil(nb / 2) and floor(nb / 2) -- with the upper and lower half of the tile instead, a
-    // tile of 128 rows kept four of the eight waves busy for as long as a full one.  16-row fragment f of wave row wm
+    // tile of nb blocks gives them ceil(nb / 2) and floor(nb / 2) (the two wave rows of a wave column share a SIMD,
+    // so the MFMA time of a short tile is the same either way; the even split evens out their LDS reads and waits).  16-row fragment f of wave row wm
     // (f < 2 * nmi, nmi = the wave's blocks, wave-uniform) starts at tile row frag_row(f).
     const int nblocks = valid / kRowBlock;
     int nmi = (wm == 0) ? (nblocks + 1) / 2 : nblocks / 2;
