@@ -73,6 +73,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--tokens", type=int, default=64, help="batch size T of the headline workload")
+    ap.add_argument("--routing", choices=["normal", "zipf", "two_experts", "balanced"], default="normal",
+                    help="router logits of the headline workload: N(0,1) (default), N(0,1) + a Zipf bias per expert, "
+                         "two experts far ahead, or exactly 2T/E rows per expert (the best case of the tiled kernels)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the other batch sizes")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end generation row")
@@ -129,6 +132,11 @@ def make_batch(torch, dev, T, seed=0, logits="normal"):
         lg = lg + torch.log(ranks / ranks.sum())[perm].to(dev)
     elif logits == "two_experts":
         lg[:, :2] += 20.0
+    elif logits == "balanced":  # token t -> experts 2t, 2t+1 (mod E): every expert gets exactly 2T/E rows
+        t = torch.arange(T, device=dev)
+        lg = torch.full_like(lg, -10.0)
+        lg[t, (2 * t) % E] = 10.0
+        lg[t, (2 * t + 1) % E] = 5.0
     return x, lg.to(torch.bfloat16)
 
 
@@ -442,7 +450,8 @@ def main():
     err_host = None if args.no_errors else host
 
     T = args.tokens
-    head = measure(torch, T, weights, args.steps, args.warmup, mode=args.mode, host=err_host, stages=True, percentiles=True)
+    head = measure(torch, T, weights, args.steps, args.warmup, logits=args.routing, mode=args.mode, host=err_host,
+                   stages=True, percentiles=True)
     roofline = w13_roofline(head)
 
     detail = []
@@ -503,7 +512,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic" if args.operands == "gaussian" else "synthetic, all-zero x and weights (diagnostic)",
         "config": {"workload": f"Mixtral-{args.shape} MoE layer T={T}: H={H} I={I} E={E} top-{TOPK} renormalised, "
-                               f"x~N(0,1), w~N(0,0.02), logits~N(0,1)",
+                               f"x~N(0,1), w~N(0,0.02), logits~N(0,1)" +
+                               ("" if args.routing == "normal" else f", routing {args.routing}"),
                    "tokens": T, "n_active_experts": head["n_active"], "mode": args.mode, "flags": MODES[args.mode],
                    "w2_dtype": "f16 copy of the bf16 weights (loader)" if MODES[args.mode] & F_W2_F16 else "bf16",
                    "max_abs_err": sig(e.get("max_abs"), 3), "mean_rel_err": sig(e.get("mean_rel"), 3),
