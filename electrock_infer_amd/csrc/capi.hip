@@ -25,10 +25,27 @@ constexpr int64_t kStreamMaxT = 64;
 constexpr int64_t kStreamW2MaxT = 8;
 // Tile height of the tiled kernels by batch size (8 experts, top-2: T/4 rows per expert on
 // average): 64-row tiles while most experts fit one of them, 128-row tiles likewise, then the
-// 256-row tiles.  Measured cross-overs on the 8x7B shape: 192 / 352 tokens.
+// 256-row tiles.  Measured cross-overs of the w13 GEMM on the 8x7B shape: 192 / 352 tokens (with N(0,1) router
+// logits the 128-row tiles stay ahead up to 470 tokens, 318 against 334 us at 448; with a Zipf bias per expert the
+// 256-row tiles win from 300 tokens, 338 against 386 us at 384: the earlier switch is kept).
 constexpr int64_t kTile64MaxT = 192;
 constexpr int64_t kTile128MaxT = 352;
-constexpr int64_t kTile128W2MaxT = 448;  // the w2 GEMM stays on 128-row tiles a little longer (156-160 against 165 us)
+// w2 GEMM.  With one row tile per expert the 256-row kernel has E x H/256 x ksplit tiles, and a launch of tiles that
+// each stream their weight rows takes whole rounds of the CUs.  Where the tiles fill their last round (8x7B: 256
+// tiles on 256 CUs) that kernel is as fast as the 128-row tiles right above the 64-row range and faster from 256
+// tokens (T=224 / 256 / 320 / 384 / 448: 145 / 149 / 150 / 154 / 158 us against 145 / 152 / 154 / 165 / 170), and far
+// ahead when the routing is uneven (router logits with a Zipf bias per expert, T=224 / 304 / 448: 170 / 190 / 230
+// against 264 / 250 / 259 us); where they do not (8x22B: 384 tiles, a round and a half) the 128-row kernel, which
+// cuts the rest of a round into narrower tiles, stays ahead up to 448 tokens (T=352: 270 against 299 us).
+constexpr int kCus = 256;  // of the GPU this library is tuned for
+constexpr int64_t kTile128W2MaxT = 448, kTile128W2MaxTFullRounds = kTile64MaxT;
+inline int64_t w2_tile128_max_tokens(int H, int E, int ksplit) {
+    const int64_t tiles = static_cast<int64_t>(E) * (H / 256) * ksplit;
+    const int64_t rounds = ceil_div(tiles, static_cast<int64_t>(kCus));
+    return tiles > 0 && tiles * 10 >= rounds * kCus * 9 ? kTile128W2MaxTFullRounds : kTile128W2MaxT;
+}
+// Above this many tokens the w2 partial sums are stored as fp16 with a float32 escape (the 256-row w2 kernel's form)
+constexpr int64_t kF32PartialsMaxT = 448;
 // Up to this many tokens router and sort share one launch (a single workgroup, whose time grows with the batch);
 // above, the two kernels (the router on many workgroups) are faster than the launch they save (8x7B layer, fused
 // against separate: T=256 473.4 / 473.9 us, T=512 552.9 / 550.0, T=1024 929 / 920, T=2048 1428 / 1408).
@@ -110,7 +127,8 @@ Plan make_plan(int64_t T, int H, int I, int E, int top_k, unsigned flags) {
     const bool bf16_act = (flags & EM_FLAG_BF16_ACT) != 0;
     pl.act_f16 = !bf16_act && (pl.use_stream || pl.use_tile);
     pl.act_pair = !bf16_act && !pl.act_f16;
-    pl.y_f16 = !(flags & EM_FLAG_F32_PARTIALS) && pl.use_tile && T > kTile128W2MaxT;
+    static_assert(kF32PartialsMaxT >= kTile128W2MaxT, "fp16 partial sums are the 256-row w2 kernel's");  // (at most)
+    pl.y_f16 = !(flags & EM_FLAG_F32_PARTIALS) && pl.use_tile && T > kF32PartialsMaxT;
     return pl;
 }
 
@@ -398,7 +416,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     const bool use_stream = pl.use_stream, use_tile = pl.use_tile;
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
         if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
-        if (T <= kTile128MaxT || (mode == 2 && T <= kTile128W2MaxT)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
+        if (T <= (mode == 1 ? kTile128MaxT : w2_tile128_max_tokens(H, E, q.ksplit))) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
         int* tickets = (flags & EM_FLAG_NO_PERSIST) ? nullptr : reinterpret_cast<int*>(ws + L.tickets_off) + (mode - 1) * 8;
         // the sort kernel clears both launches' counters; a call that skips it (stage timing) clears them here
         return launch_gemm_tile(q, seg_begin, mode, tickets, (flags & EM_FLAG_SKIP_ALIGN) != 0, s);

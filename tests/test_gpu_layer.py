@@ -637,7 +637,7 @@ def test_layer_mid_kernel_many_column_tiles(T, I, routing):
     check_outputs(f"wideI{I}_T{T}_{routing}", out_f32.cpu(), out_bf16.cpu(), ref, out_def.cpu())
 
 
-@pytest.mark.parametrize("T", [8, 9, 16, 17, 63, 64, 191, 192, 193, 351, 352, 353, 447, 448, 449, 895, 896, 897,
+@pytest.mark.parametrize("T", [8, 9, 16, 17, 63, 64, 191, 192, 193, 255, 256, 257, 351, 352, 353, 447, 448, 449, 895, 896, 897,
                                1023, 1024, 1025, 1279, 1280, 1281, 2047, 2048, 2049])
 def test_layer_at_every_kernel_switch(T):
     """The batch sizes on both sides of every point where the layer changes kernels, K slices, sorted block,
@@ -725,7 +725,7 @@ def _drawn_case(seed):
     H = int(rng.choice([64, 136, 256, 320, 512, 768, 1024, 1280, 2048]))
     I = int(rng.choice([64, 200, 256, 384, 512, 640, 1024, 1152, 1536, 2048, 3584]))
     E, k = [(8, 2), (8, 2), (8, 2), (8, 1), (4, 2), (16, 2), (2, 2), (32, 3), (64, 6)][int(rng.integers(9))]
-    T = int(rng.choice([1, 2, 5, 8, 9, 16, 17, 31, 48, 64, 65, 100, 129, 192, 193, 250, 352, 353, 449, 600, 897, 1300, 2049, 2100]))
+    T = int(rng.choice([1, 2, 5, 8, 9, 16, 17, 31, 48, 64, 65, 100, 129, 192, 193, 250, 288, 352, 353, 449, 600, 897, 1300, 2049, 2100]))
     routing = ["normal", "zipf", "two_experts"][int(rng.integers(3))]
     logits_dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(3))]
     return H, I, E, k, T, routing, logits_dtype, bool(rng.integers(2))
