@@ -23,26 +23,34 @@ constexpr int64_t kStreamMaxT = 64;
 // 10 % (8x7B; T=16: 138 against 146 us, T=12: 121 against 126, T=8: equal, T=5: 98 against 90) and is 20 % ahead
 // throughout on the 8x22B shape.
 constexpr int64_t kStreamW2MaxT = 8;
-// Tile height of the tiled kernels by batch size (8 experts, top-2: T/4 rows per expert on
-// average): 64-row tiles while most experts fit one of them, 128-row tiles likewise, then the
-// 256-row tiles.  Measured cross-overs of the w13 GEMM on the 8x7B shape: 192 / 352 tokens (with N(0,1) router
-// logits the 128-row tiles stay ahead up to 470 tokens, 318 against 334 us at 448; with a Zipf bias per expert the
-// 256-row tiles win from 300 tokens, 338 against 386 us at 384: the earlier switch is kept).
-constexpr int64_t kTile64MaxT = 192;
-constexpr int64_t kTile128MaxT = 352;
-// w2 GEMM.  With one row tile per expert the 256-row kernel has E x H/256 x ksplit tiles, and a launch of tiles that
-// each stream their weight rows takes whole rounds of the CUs.  Where the tiles fill their last round (8x7B: 256
-// tiles on 256 CUs) that kernel is as fast as the 128-row tiles right above the 64-row range and faster from 256
-// tokens (T=224 / 256 / 320 / 384 / 448: 145 / 149 / 150 / 154 / 158 us against 145 / 152 / 154 / 165 / 170), and far
-// ahead when the routing is uneven (router logits with a Zipf bias per expert, T=224 / 304 / 448: 170 / 190 / 230
-// against 264 / 250 / 259 us); where they do not (8x22B: 384 tiles, a round and a half) the 128-row kernel, which
-// cuts the rest of a round into narrower tiles, stays ahead up to 448 tokens (T=352: 270 against 299 us).
+// Tile height of the tiled kernels above the streaming range (8 experts, top-2: T/4 rows per expert on average).
+// Every tile streams the weight rows of its columns once, whatever its height, so a launch takes as many rounds of
+// the CUs as its tiles make.  The 256-row kernel hands its tiles out through a queue and has one row tile per expert
+// up to about 1000 tokens: E x (column tiles) x (K slices) tiles.
+//   * Where these fill their last round (w2 of 8x7B: 256 tiles on 256 CUs; w13 of 8x22B: 1024) it is the kernel from
+//     65 tokens on: as fast as the 128-row tiles with even routing (8x7B w2, T=128 / 224 / 320 / 448: 147 / 145 / 150 /
+//     158 us against 146 / 145 / 154 / 170; 8x22B w13, T=128: 480 against 478 us) and far ahead with uneven routing,
+//     where experts outgrow a 128-row tile long before the average does (router logits with a Zipf bias per expert,
+//     8x7B w2 T=160 / 224 / 448: 164 / 170 / 230 us against 243 / 264 / 259; 8x22B w13 T=128: 490 against 525).
+//   * Where they leave a round part empty (w13 of 8x7B: 896 tiles, three and a half rounds; w2 of 8x22B: 384) the
+//     128-row kernel stays: it cuts the rest of a round into narrower tiles, a round of half the length (8x7B w13
+//     T=128 / 256: 291 / 293 us against 308 / 309), up to the batch sizes where most experts still fit one of its
+//     tiles: 352 tokens for the w13 GEMM (with even routing it would stay ahead up to 470 tokens, 318 against 334 us
+//     at 448; with the Zipf bias the 256-row tiles win from 200 tokens, 313 against 359 us at 224: the earlier switch
+//     is kept), 448 for the w2 GEMM (8x22B T=352: 270 against 299 us).
+// 64-row tiles are as fast as 128-row tiles with even routing from 65 to 192 tokens and a fifth slower with the Zipf
+// bias (8x7B layer, T=128: 0.451 / 0.451 ms even, 0.597 / 0.491 ms uneven): the large-batch path does not use them.
 constexpr int kCus = 256;  // of the GPU this library is tuned for
-constexpr int64_t kTile128W2MaxT = 448, kTile128W2MaxTFullRounds = kTile64MaxT;
-inline int64_t w2_tile128_max_tokens(int H, int E, int ksplit) {
-    const int64_t tiles = static_cast<int64_t>(E) * (H / 256) * ksplit;
+constexpr int64_t kTile128MaxT = 352, kTile128W2MaxT = 448;
+inline bool tiles_fill_rounds(int64_t tiles) {
     const int64_t rounds = ceil_div(tiles, static_cast<int64_t>(kCus));
-    return tiles > 0 && tiles * 10 >= rounds * kCus * 9 ? kTile128W2MaxTFullRounds : kTile128W2MaxT;
+    return tiles > 0 && tiles * 10 >= rounds * kCus * 9;
+}
+// mode 1: w13 GEMM, 2: w2 GEMM; batches up to the returned size run on 128-row tiles
+inline int64_t tile128_max_tokens(int mode, int H, int I, int E, int ksplit) {
+    const int64_t tiles = static_cast<int64_t>(E) * (mode == 1 ? I / 128 : static_cast<int64_t>(H / 256) * ksplit);
+    if (tiles_fill_rounds(tiles)) return kStreamMaxT;
+    return mode == 1 ? kTile128MaxT : kTile128W2MaxT;
 }
 // Above this many tokens the w2 partial sums are stored as fp16 with a float32 escape (the 256-row w2 kernel's form)
 constexpr int64_t kF32PartialsMaxT = 448;
@@ -415,8 +423,7 @@ int moe_forward_impl(const void* x, const void* router_logits, int logits_dtype,
     }
     const bool use_stream = pl.use_stream, use_tile = pl.use_tile;
     auto tile_gemm = [&](const MoeProblem& q, int mode) {
-        if (T <= kTile64MaxT) return launch_gemm_tile_mid(q, seg_begin, mode, 64, s);
-        if (T <= (mode == 1 ? kTile128MaxT : w2_tile128_max_tokens(H, E, q.ksplit))) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
+        if (T <= tile128_max_tokens(mode, H, I, E, q.ksplit)) return launch_gemm_tile_mid(q, seg_begin, mode, 128, s);
         int* tickets = (flags & EM_FLAG_NO_PERSIST) ? nullptr : reinterpret_cast<int*>(ws + L.tickets_off) + (mode - 1) * 8;
         // the sort kernel clears both launches' counters; a call that skips it (stage timing) clears them here
         return launch_gemm_tile(q, seg_begin, mode, tickets, (flags & EM_FLAG_SKIP_ALIGN) != 0, s);

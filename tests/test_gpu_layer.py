@@ -148,9 +148,10 @@ def mixtral_8x7b():
     return {"x": x, "lg": lg, "w13": w13, "w2": w2, "w13_cpu": w13.cpu(), "w2_cpu": w2.cpu()}
 
 
-@pytest.mark.parametrize("T", [1, 8, 32, 64, 256])
+@pytest.mark.parametrize("T", [1, 8, 32, 64, 65, 130, 256])
 def test_layer_8x7b_decode(mixtral_8x7b, T):
-    """Configuration 2: H=4096, I=14336, E=8, top-2, bf16, decode batch sizes."""
+    """Configuration 2: H=4096, I=14336, E=8, top-2, bf16, decode batch sizes (from 65 tokens the w2 GEMM of this
+    shape runs on the 256-row kernel)."""
     announce(f"layer 8x7B decode T={T}")
     m = mixtral_8x7b
     x, lg = m["x"][:T].contiguous(), m["lg"][:T].contiguous()
@@ -161,6 +162,24 @@ def test_layer_8x7b_decode(mixtral_8x7b, T):
     rows = list(range(T)) if T <= 64 else list(range(0, T, 4))
     ref = oracle_rows(x, lg, m["w13_cpu"], m["w2_cpu"], rows)
     check_outputs(f"8x7b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_def[rows].cpu(), def_bf16[rows].cpu())
+
+
+@pytest.mark.parametrize("T", [65, 200, 448])
+def test_layer_8x7b_small_batches_with_two_busy_experts(mixtral_8x7b, T):
+    """Small batches whose tokens all pick experts 0 and 1: six experts without rows, two with T rows each, on the
+    kernels that even routing would give a few dozen rows per expert."""
+    announce(f"layer 8x7B T={T}, all tokens to experts 0 and 1")
+    m = mixtral_8x7b
+    lg = m["lg"][:T].float()
+    lg[:, :2] += 20.0
+    lg = lg.to(torch.bfloat16).contiguous()
+    x = m["x"][:T].contiguous()
+    out_f32, out_bf16 = run_both(x, lg, m["w13"], m["w2"])
+    out_def = run_default(x, lg, m["w13"], m["w2"])
+    check_routing(get_workspace(DEV, T, 4096, 14336, 8, 2), lg.float().cpu(), T)
+    rows = list(range(0, T, max(1, T // 48)))
+    ref = oracle_rows(x, lg, m["w13_cpu"], m["w2_cpu"], rows)
+    check_outputs(f"8x7b_T{T}_two_experts", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_def[rows].cpu())
 
 
 @pytest.mark.parametrize("logits", ["normal", "zipf", "two_experts"])
