@@ -233,8 +233,8 @@ int tile_row_block();
 bool tile_supported(const MoeProblem& p);
 int launch_gemm_tile(const MoeProblem& p, const int32_t* seg_begin, int mode, int* tickets /* 8 ints or null */,
                      bool clear_tickets /* they were not cleared by the sort in front */, hipStream_t s);                                                               // 256-row tiles
-bool tile_mid_supported(const MoeProblem& p);                                                      // 64- / 128-row tiles
-int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile /* 64 | 128 */,
+bool tile_mid_supported(const MoeProblem& p);                                                      // 128- / 64-row tiles
+int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile /* 128 | w2: 64 */,
                          hipStream_t s);
 int launch_combine(const MoeProblem& p, void* out, int out_f32, hipStream_t s);
 

@@ -4,8 +4,8 @@
 // This kernel is the 256-row tiled kernel cut down in M, and where it pays in N, so that
 // LDS holds a deeper copy ring and the tiles fill whole rounds of CUs:
 //
-//   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile of up to 64 (MI = 1) or 128 (MI = 2)
-//              sorted rows x NT = 128 or 256 weight rows; wave sub-tile (32 MI) x (NT / 4) as
+//   workgroup  512 threads = 8 waves as 2 (M) x 4 (N); tile of up to 128 (MI = 2) or, for the w2 GEMM of decode
+//              batches, 64 (MI = 1) sorted rows x NT = 128 or 256 weight rows; wave sub-tile (32 MI) x (NT / 4) as
 //              2 MI x NT / 64 accumulators of v_mfma_f32_16x16x32_bf16
 //   ring       S stages of 8 MI KB of token rows + NT / 8 KB of weight rows (K step 64), as many
 //              as fit 160 KB (3 .. 6), all but one in flight while that one is multiplied:
@@ -414,11 +414,11 @@ bool tile_mid_supported(const MoeProblem& p) {
            p.I % (p.ksplit * kTK) == 0;
 }
 
-// rows_per_tile: 64 or 128
+// rows_per_tile: 128, or 64 for the w2 GEMM (decode batches; the w13 GEMM has no use for 64-row tiles: above the
+// streaming kernel's range they are no faster than 128-row tiles with even routing and slower with uneven routing)
 int launch_gemm_tile_mid(const MoeProblem& p, const int32_t* seg_begin, int mode, int rows_per_tile, hipStream_t s) {
-    if (!tile_mid_supported(p)) return EM_ERR_UNSUPPORTED;
-    if (mode == 1 && p.act_f16) return rows_per_tile == 64 ? launch_mid<1, 1, true>(p, seg_begin, s) : launch_mid<1, 2, true>(p, seg_begin, s);
-    if (mode == 1) return rows_per_tile == 64 ? launch_mid<1, 1, false>(p, seg_begin, s) : launch_mid<1, 2, false>(p, seg_begin, s);
+    if (!tile_mid_supported(p) || (rows_per_tile != 128 && !(mode == 2 && rows_per_tile == 64))) return EM_ERR_UNSUPPORTED;
+    if (mode == 1) return p.act_f16 ? launch_mid<1, 2, true>(p, seg_begin, s) : launch_mid<1, 2, false>(p, seg_begin, s);
     if (p.act_f16) return rows_per_tile == 64 ? launch_mid<2, 1, true>(p, seg_begin, s) : launch_mid<2, 2, true>(p, seg_begin, s);
     return rows_per_tile == 64 ? launch_mid<2, 1, false>(p, seg_begin, s) : launch_mid<2, 2, false>(p, seg_begin, s);
 }
