@@ -304,13 +304,17 @@ def test_layer_8x7b_float16_w2(mixtral_8x7b):
 
 
 def test_layer_8x22b_shape():
-    """Configuration 5: H=6144, I=16384; T in {1, 64} in full, T=4096 on sampled tokens."""
+    """Configuration 5: H=6144, I=16384; T in {1, 64} in full, T=100 (the w13 GEMM of this shape runs on the 256-row
+    kernel from 65 tokens, the w2 GEMM on 128-row tiles), with even routing and with all tokens on experts 0 and 1, and
+    T=4096 on sampled tokens."""
     announce("building 8x22B-shaped weights")
     x, lg, w13, w2 = gpu_inputs(4096, 6144, 16384, seed=1)
     w13_cpu, w2_cpu = w13.cpu(), w2.cpu()
-    for T in (1, 64, 4096):
+    lg_two = lg[:100].float()
+    lg_two[:, :2] += 20.0
+    for T, lt in ((1, lg[:1]), (64, lg[:64]), (100, lg[:100]), (100, lg_two.to(torch.bfloat16)), (4096, lg)):
         announce(f"layer 8x22B T={T}")
-        xt, lt = x[:T].contiguous(), lg[:T].contiguous()
+        xt, lt = x[:T].contiguous(), lt.contiguous()
         out_f32, out_bf16 = run_both(xt, lt, w13, w2)
         out_def = run_default(xt, lt, w13, w2)
         def_bf16 = fused_experts(xt, w13, w2, lt, 2)
