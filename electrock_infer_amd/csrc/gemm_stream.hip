@@ -30,7 +30,10 @@ constexpr int kWaves = 4;
 constexpr int kStep = 64;                 // K elements per step (128 B per weight row)
 constexpr int kRows = 64;                 // weight rows per workgroup
 constexpr int kPitch = kStep * 2 + 16;    // 144 B
-constexpr int kMaxF = 2;                  // 16-row token fragments per pass
+constexpr int kMaxF = 2;                  // 16-row token fragments of a pass whose rows are fetched two steps ahead
+// further fragments of the same pass, fetched in the step that uses them (w13 GEMM: up to 64 tokens an expert has at
+// most 64 rows; the w2 GEMM runs here up to 8 tokens only, one fragment per expert, and keeps its registers)
+template <int MODE> struct Extra { static constexpr int kMaxX = MODE == 1 ? 2 : 0; };
 
 __device__ __forceinline__ u32x4_t ld16(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 // Weights are read exactly once per call: a non-temporal load keeps the stream from
@@ -48,6 +51,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
                                                                      const int32_t* __restrict__ seg_begin,
                                                                      int tiles_per_expert, int kslice) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kWaves][kRows * kPitch];
+    constexpr int kMaxX = Extra<MODE>::kMaxX;
+    constexpr int kPassF = kMaxF + kMaxX;  // fragments per pass over the weight rows
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -89,15 +94,21 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
     const int r16 = lane & 15;
     const int kq = lane >> 4;
 
-    for (int f0 = 0; f0 < nfrag_total; f0 += kMaxF) {
-        const int nf = (nfrag_total - f0 < kMaxF) ? nfrag_total - f0 : kMaxF;
+    // A pass streams the workgroup's weight rows once for up to kPassF fragments.  With even routing a decode batch
+    // has one or two fragments per expert: their token rows are prefetched as deep as the weights.  An expert that the
+    // routing favours brings a third and fourth; their rows (L2 hits) are fetched in the step that multiplies them, which
+    // costs that workgroup part of its prefetch distance but not a second pass over the weights.
+    for (int f0 = 0; f0 < nfrag_total; f0 += kPassF) {
+        const int nall = (nfrag_total - f0 < kPassF) ? nfrag_total - f0 : kPassF;
+        const int nf = nall < kMaxF ? nall : kMaxF;
+        const int nx = nall - nf;  // workgroup-uniform
 
         // token rows of this lane (operand layout: row r16 of each fragment)
-        const uint16_t* arow[kMaxF];
+        const uint16_t* arow[kPassF];
 #pragma unroll
-        for (int f = 0; f < kMaxF; ++f) {
+        for (int f = 0; f < kPassF; ++f) {
             arow[f] = nullptr;
-            if (f < nf) {
+            if (f < nall) {
                 const int pos = seg + (f0 + f) * 16 + r16;
                 if (MODE == 1) {
                     const int slot = p.sorted_ids[pos];
@@ -108,9 +119,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
             }
         }
 
-        f32x4_t acc[kMaxF][4];
+        f32x4_t acc[kPassF][4];
 #pragma unroll
-        for (int f = 0; f < kMaxF; ++f)
+        for (int f = 0; f < kPassF; ++f)
 #pragma unroll
             for (int g = 0; g < 4; ++g) acc[f][g] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -127,7 +138,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
                     a[f][ks] = (arow[f] != nullptr) ? ld16(arow[f] + koff + ks * 32) : u32x4_t{0, 0, 0, 0};
                 }
         };
-        auto consume = [&](u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][kAW]) {
+        auto consume = [&](int s, u32x4_t(&b)[8], u32x4_t(&a)[kMaxF][kAW]) {
+            u32x4_t ax[kMaxX > 0 ? kMaxX : 1][kAW];
+            if (kMaxX > 0 && nx > 0) {
+#pragma unroll
+                for (int f = 0; f < kMaxX; ++f)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+                        ax[f][ks] = (arow[kMaxF + f] != nullptr) ? ld16(arow[kMaxF + f] + s * kStep + ks * 32) : u32x4_t{0, 0, 0, 0};
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 *reinterpret_cast<u32x4_t*>(my + (i * 8 + lrow) * kPitch + lchunk * 16) = b[i];
@@ -161,56 +180,80 @@ __global__ __launch_bounds__(kWaves * 64, 2) void gemm_stream_kernel(MoeProblem 
                         }
                     }
                 }
+                if (kMaxX > 0 && nx > 0) {
+#pragma unroll
+                    for (int f = 0; f < kMaxX; ++f) {
+                        if (f < nx) {
+                            if (F16) {
+                                f16x8_t af;
+                                __builtin_memcpy(&af, &ax[f][ks], 16);
+#pragma unroll
+                                for (int g = 0; g < 4; ++g)
+                                    acc[kMaxF + f][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, hf[g], acc[kMaxF + f][g], 0, 0, 0);
+                            } else {
+                                bf16x8_t af;
+                                __builtin_memcpy(&af, &ax[f][ks], 16);
+#pragma unroll
+                                for (int g = 0; g < 4; ++g)
+                                    acc[kMaxF + f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[g], acc[kMaxF + f][g], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
             }
         };
 
         if (nsteps > 0) issue(0, b0, a0);
         if (nsteps > 1) issue(1, b1, a1);
         for (int s = 0; s < nsteps; s += 2) {
-            consume(b0, a0);
+            consume(s, b0, a0);
             if (s + 2 < nsteps) issue(s + 2, b0, a0);
             if (s + 1 < nsteps) {
-                consume(b1, a1);
+                consume(s + 1, b1, a1);
                 if (s + 3 < nsteps) issue(s + 3, b1, a1);
             }
         }
 
-        // ---- meet the four K-slice partials in LDS (reusing the staging tiles) ----
-        __syncthreads();
-        f32x4_t* red = reinterpret_cast<f32x4_t*>(&lds[0][0]);  // [wave][f][g][lane]
+        // ---- meet the four K-slice partials in LDS (reusing the staging tiles), kMaxF fragments at a time ----
+        for (int h0 = 0; h0 < nall; h0 += kMaxF) {
+            const int nh = (nall - h0 < kMaxF) ? nall - h0 : kMaxF;
+            __syncthreads();
+            f32x4_t* red = reinterpret_cast<f32x4_t*>(&lds[0][0]);  // [wave][f][g][lane]
 #pragma unroll
-        for (int f = 0; f < kMaxF; ++f)
+            for (int f = 0; f < kMaxF; ++f)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) red[((wave * kMaxF + f) * 4 + g) * 64 + lane] = acc[f][g];
-        __syncthreads();
-        auto total = [&](int f, int g) {
-            f32x4_t s = red[((0 * kMaxF + f) * 4 + g) * 64 + lane];
+                for (int g = 0; g < 4; ++g)
+                    red[((wave * kMaxF + f) * 4 + g) * 64 + lane] = (kMaxX == 0 || h0 == 0) ? acc[f][g] : acc[(kMaxF + f) % kPassF][g];
+            __syncthreads();
+            auto total = [&](int f, int g) {
+                f32x4_t t = red[((0 * kMaxF + f) * 4 + g) * 64 + lane];
 #pragma unroll
-            for (int w = 1; w < kWaves; ++w) s += red[((w * kMaxF + f) * 4 + g) * 64 + lane];
-            return s;
-        };
-        if (MODE == 1) {
-            if (wave < 2) {
-                const int j = tile * 32 + wave * 16 + r16;
-                for (int f = 0; f < nf; ++f) {
-                    const f32x4_t g = total(f, wave);
-                    const f32x4_t u = total(f, 2 + wave);
+                for (int w = 1; w < kWaves; ++w) t += red[((w * kMaxF + f) * 4 + g) * 64 + lane];
+                return t;
+            };
+            if (MODE == 1) {
+                if (wave < 2) {
+                    const int j = tile * 32 + wave * 16 + r16;
+                    for (int f = 0; f < nh; ++f) {
+                        const f32x4_t g = total(f, wave);
+                        const f32x4_t u = total(f, 2 + wave);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const int64_t row = seg + (f0 + f) * 16 + kq * 4 + v;
-                        store_act(p, row * p.I + j, silu_mul(g[v], u[v]));
+                        for (int v = 0; v < 4; ++v) {
+                            const int64_t row = seg + (f0 + h0 + f) * 16 + kq * 4 + v;
+                            store_act(p, row * p.I + j, silu_mul(g[v], u[v]));
+                        }
                     }
                 }
-            }
-        } else {
-            float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H;
-            const int n = tile * kRows + wave * 16 + r16;
-            for (int f = 0; f < nf; ++f) {
-                const f32x4_t t = total(f, wave);
+            } else {
+                float* ybase = p.y + static_cast<int64_t>(blockIdx.y) * p.T * p.top_k * p.H;
+                const int n = tile * kRows + wave * 16 + r16;
+                for (int f = 0; f < nh; ++f) {
+                    const f32x4_t t = total(f, wave);
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int slot = p.sorted_ids[seg + (f0 + f) * 16 + kq * 4 + v];
-                    if (slot >= 0) ybase[static_cast<int64_t>(slot) * p.H + n] = t[v];
+                    for (int v = 0; v < 4; ++v) {
+                        const int slot = p.sorted_ids[seg + (f0 + h0 + f) * 16 + kq * 4 + v];
+                        if (slot >= 0) ybase[static_cast<int64_t>(slot) * p.H + n] = t[v];
+                    }
                 }
             }
         }

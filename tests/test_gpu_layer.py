@@ -164,10 +164,26 @@ def test_layer_8x7b_decode(mixtral_8x7b, T):
     check_outputs(f"8x7b_T{T}", out_f32[rows].cpu(), out_bf16[rows].cpu(), ref, out_def[rows].cpu(), def_bf16[rows].cpu())
 
 
-@pytest.mark.parametrize("T", [65, 200, 448])
+@pytest.mark.parametrize("T", [17, 33, 48, 64])
+def test_layer_config1_shape_two_busy_experts_in_a_decode_batch(T):
+    """Decode batches whose tokens all pick experts 0 and 1: T rows per expert, i.e. two to four 16-row fragments in
+    one pass of the streaming kernel over the weight rows (even routing gives one or two); every row against the
+    oracle."""
+    announce(f"layer C1-shape T={T}, all tokens to experts 0 and 1")
+    x, lg, w13, w2 = O.make_inputs(T, 256, 512, seed=T, logits="two_experts")
+    ref = O.moe_layer_fp32(x, lg, w13, w2)
+    xd, lgd, w13d, w2d = (t.to(DEV) for t in (x, lg, w13, w2))
+    out_f32, out_bf16 = run_both(xd, lgd, w13d, w2d)
+    out_def = run_default(xd, lgd, w13d, w2d)
+    check_routing(get_workspace(DEV, T, 256, 512, 8, 2), lg.float(), T)
+    check_outputs(f"c1_T{T}_two_experts", out_f32.cpu(), out_bf16.cpu(), ref, out_def.cpu())
+
+
+@pytest.mark.parametrize("T", [40, 64, 65, 200, 448])
 def test_layer_8x7b_small_batches_with_two_busy_experts(mixtral_8x7b, T):
     """Small batches whose tokens all pick experts 0 and 1: six experts without rows, two with T rows each, on the
-    kernels that even routing would give a few dozen rows per expert."""
+    kernels that even routing would give a few dozen rows per expert (up to 64 tokens: three and four fragments in one
+    pass of the streaming kernel)."""
     announce(f"layer 8x7B T={T}, all tokens to experts 0 and 1")
     m = mixtral_8x7b
     lg = m["lg"][:T].float()
