@@ -2,7 +2,7 @@
 """Benchmark of the Mixtral MoE layer on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T] [--shape 8x7b|8x22b] [--mode MODE]
-                    [--no-cpu] [--no-table] [--no-e2e] [--detail FILE]
+                    [--routing normal|zipf|two_experts|balanced] [--no-cpu] [--no-table] [--no-e2e] [--detail FILE]
 
 A "step" is one call of the layer (router, expert sort, w13 GEMM + SiLU*mul,
 w2 GEMM, top-k combine) on one batch of T tokens resident in HBM.  The headline
@@ -463,6 +463,11 @@ def main():
         for t in ((1, 8, 32, 64, 256, 512, 1024, 2048) if args.shape == "8x7b" else (1, 64)):
             if t != T or args.mode != "default_f32out":
                 detail.append(measure(torch, t, weights, half_steps if t <= 256 else 30, half_warm, host=err_host))
+        if args.shape == "8x7b":
+            # uneven routing at decode and mid sizes (the kernels there are chosen by batch size: an expert far above the
+            # average must not cost a second pass over its weights)
+            for t in (64, 256):
+                detail.append(measure(torch, t, weights, half_steps, half_warm, logits="zipf", host=err_host))
         for lgk in (("normal", "zipf", "two_experts") if args.shape == "8x7b" else ("normal",)):
             detail.append(measure(torch, big, weights, 20, 5, logits=lgk, host=err_host, stages=lgk == "normal"))
             if lgk == "normal":
