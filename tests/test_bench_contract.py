@@ -49,6 +49,28 @@ def test_rows_of_the_printed_line_stay_short():
     assert bench.MODES["default_f32out"] == bench.F_W2_F16 | bench.F_OUT_F32 and bench.MODES["default"] == bench.F_W2_F16
 
 
+def test_routing_kinds_of_the_synthetic_batch():
+    """`balanced` gives every expert exactly 2T/E rows (the tiled kernels' best case), `two_experts` sends every token
+    to experts 0 and 1, `zipf` favours one expert; x is the same whatever the routing."""
+    import torch
+    sys.path.insert(0, ROOT)
+    import bench
+    dev, T = torch.device("cpu"), 256
+    x0, lg = bench.make_batch(torch, dev, T, logits="normal")
+    assert x0.shape == (T, bench.H) and lg.shape == (T, bench.E) and lg.dtype == torch.bfloat16
+    counts = {}
+    for kind in ("normal", "zipf", "two_experts", "balanced"):
+        x, lg = bench.make_batch(torch, dev, T, logits=kind)
+        assert torch.equal(x, x0)
+        ids = lg.float().topk(bench.TOPK, dim=1).indices
+        counts[kind] = torch.bincount(ids.flatten(), minlength=bench.E)
+        assert int(counts[kind].sum()) == T * bench.TOPK
+    assert counts["balanced"].tolist() == [T * bench.TOPK // bench.E] * bench.E
+    assert counts["two_experts"].tolist() == [T, T] + [0] * (bench.E - 2)
+    assert int(counts["zipf"].max()) > 2 * T * bench.TOPK // bench.E      # the busiest expert: more than twice its share
+    assert int(counts["normal"].max()) < 2 * T * bench.TOPK // bench.E
+
+
 @pytest.mark.gpu
 def test_json_line_of_a_short_run():
     p = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "2", "--no-table", "--no-cpu"],
